@@ -1,0 +1,64 @@
+"""Pins oracle/attn_tiled.c (the C restatement of the reference's tiled kernels)
+against oracle/eager_ref.py and against the transformers golden vectors."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import eager_ref as E
+from oracle import tiled as T
+
+SCALE = 0.125
+
+CASES = [
+    # S, window, seqlens, q_offset, Skv
+    (100, None, None, 0, None),
+    (130, 32, None, 0, None),
+    (200, 128, None, 0, None),
+    (96, 17, [50, 96], 0, None),
+    (70, None, [1, 70], 0, None),
+    (40, None, None, 24, 64),
+    (40, 16, None, 24, 64),
+]
+
+
+@pytest.mark.parametrize("s,w,sl,qo,skv", CASES)
+def test_tiled_matches_eager(s, w, sl, qo, skv):
+    b = len(sl) if sl else 1
+    q, k, v, sinks, d_out = E.make_inputs(21, b, 8, 2, s, 64, skv=skv)
+    dbl = [t.double() for t in (q, k, v, sinks, d_out)]
+    out, dq, dk, dv, ds = E.eager_attention_grads(*dbl, SCALE, w, qo, sl)
+    lse = E.logsumexp_rows(dbl[0], dbl[1], dbl[3], SCALE, w, qo, sl)
+    o2, lse2 = T.tiled_fwd(q, k, v, sinks, SCALE, w, qo, sl)
+    dq2, dk2, dv2, ds2, delta = T.tiled_bwd(q, k, v, sinks, o2, lse2, d_out, SCALE, w, qo, sl)
+    for name, a, b_ in (("o", out, o2), ("lse", lse, lse2), ("dq", dq, dq2), ("dk", dk, dk2),
+                        ("dv", dv, dv2), ("ds", ds, ds2)):
+        assert torch.allclose(a.float(), b_, atol=3e-6, rtol=1e-5), (name, float((a.float() - b_).abs().max()))
+    assert torch.allclose(delta, (out * dbl[4]).sum(-1).permute(0, 2, 1).float(), atol=3e-6)
+
+
+def test_tiled_matches_transformers_golden(golden_dir):
+    z = np.load(os.path.join(golden_dir, "tiny_win8.npz"))
+    q, k, v, sinks, d_out = E.make_inputs(int(z["seed"]), 1, 8, 2, 64, 64)
+    o, lse = T.tiled_fwd(q, k, v, sinks, SCALE, 8)
+    dq, dk, dv, ds, _ = T.tiled_bwd(q, k, v, sinks, o, lse, d_out, SCALE, 8)
+    for name, mine in (("out", o), ("dq", dq), ("dk", dk), ("dv", dv), ("dsinks", ds)):
+        assert np.allclose(mine.numpy(), z[name], rtol=1e-4, atol=2e-5), name
+
+
+def test_null_sinks_is_zero_logit():
+    q, k, v, _, _ = E.make_inputs(22, 1, 4, 2, 30, 64)
+    a, la = T.tiled_fwd(q, k, v, None, SCALE)
+    b_, lb = T.tiled_fwd(q, k, v, torch.zeros(4), SCALE)
+    assert torch.equal(a, b_) and torch.equal(la, lb)
+
+
+def test_padded_rows_are_inert():
+    q, k, v, sinks, d_out = E.make_inputs(23, 2, 4, 2, 40, 64)
+    sl = [13, 40]
+    o, lse = T.tiled_fwd(q, k, v, sinks, SCALE, None, 0, sl)
+    assert torch.all(o[0, 13:] == 0)
+    assert torch.allclose(lse[0, :, 13:], sinks.view(-1, 1).expand(4, 27))
+    dq, dk, dv, ds, _ = T.tiled_bwd(q, k, v, sinks, o, lse, d_out, SCALE, None, 0, sl)
+    assert torch.all(dq[0, :, 13:] == 0) and torch.all(dk[0, :, 13:] == 0) and torch.all(dv[0, :, 13:] == 0)
