@@ -1,0 +1,148 @@
+/*
+ * gptoss_attn.h -- C ABI of the MI355X (gfx950) GPT-OSS flash-attention library.
+ *
+ * The reference project has no native layer: its device code is three Triton
+ * kernels launched from a torch.autograd.Function (attention_kernel.py:220-344).
+ * Each entry point below names the reference code it stands in for, so a
+ * maintainer can bind it (ctypes, cffi, a torch custom op) at the same place.
+ *
+ * Conventions
+ *   - plain pointers and sizes only; no torch, no HIP types (the stream is passed
+ *     as a void* holding a hipStream_t; NULL is the default stream);
+ *   - every buffer is owned by the caller; the library allocates nothing and
+ *     keeps no mutable global state, so calls on different streams are
+ *     independent;
+ *   - launches are asynchronous on `stream`; no entry point synchronises;
+ *   - outputs need no pre-zeroing (the reference needs dk/dv/dsinks zeroed,
+ *     attention_kernel.py:296-298; this library writes every element once);
+ *   - return value: 0 ok; negative = argument error (table below), checked on
+ *     the host before anything is launched; positive = the hipError_t of a
+ *     failed launch.  No C++ exception crosses the boundary.
+ *
+ * Tensors (element strides, innermost head_dim stride fixed at 1):
+ *   q, dq        (B, H, Sq, D)     query heads
+ *   k, v, dk, dv (B, G, Skv, D)    KV heads; query head h reads KV head h/(H/G)
+ *                                  (attention_kernel.py:36,152)
+ *   o, d_o       (B, Sq, H, D) by default in the caller's view, but addressed
+ *                through the same (b, h, s) stride triple, so any layout works
+ *   lse, delta   (B, H, Sq) fp32 contiguous
+ *   sinks, dsinks (H,) fp32;  sinks == NULL means a sink logit of 0, as in the
+ *                reference (attention_kernel.py:39-42)
+ *   seqlens      (B,) int32 or NULL: right-padding lengths.  Keys at or beyond
+ *                seqlens[b] are invisible; query rows at or beyond it produce
+ *                O = 0, lse = sink and contribute no gradient.
+ * Visibility of key j to the query at absolute position p = q_offset + i:
+ *   j <= p  and  (window == 0 or j > p - window)      (attention_kernel.py:68,71)
+ */
+#ifndef GPTOSS_ATTN_H
+#define GPTOSS_ATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GPTOSS_ATTN_ABI_VERSION 1
+
+enum gptoss_attn_dtype {
+    GPTOSS_ATTN_BF16 = 0, /* 2-byte bfloat16 tensors, fp32 accumulation */
+    GPTOSS_ATTN_FP32 = 1  /* 4-byte float tensors (the reference's fp32 mode) */
+};
+
+enum gptoss_attn_status {
+    GPTOSS_ATTN_OK = 0,
+    GPTOSS_ATTN_ERR_NULL_PARAMS = -1,   /* params pointer is NULL */
+    GPTOSS_ATTN_ERR_NULL_TENSOR = -2,   /* a required tensor pointer is NULL */
+    GPTOSS_ATTN_ERR_HEAD_DIM = -3,      /* D != 64 */
+    GPTOSS_ATTN_ERR_HEADS = -4,         /* H <= 0, G <= 0 or H % G != 0 */
+    GPTOSS_ATTN_ERR_SHAPE = -5,         /* B, Sq or Skv <= 0, window < 0, q_offset < 0 */
+    GPTOSS_ATTN_ERR_DTYPE = -6,         /* dtype not in gptoss_attn_dtype */
+    GPTOSS_ATTN_ERR_ALIGNMENT = -7,     /* a tensor base or stride breaks 16-byte row alignment */
+    GPTOSS_ATTN_ERR_STRIDE = -8,        /* a sequence stride smaller than D */
+    GPTOSS_ATTN_ERR_ABI = -9            /* struct_size does not match this library */
+};
+
+/* (batch, head, sequence) strides in elements. */
+typedef struct gptoss_attn_strides {
+    int64_t b, h, s;
+} gptoss_attn_strides;
+
+typedef struct gptoss_attn_params {
+    uint32_t struct_size;   /* sizeof(gptoss_attn_params), checked by every call */
+    int32_t dtype;          /* gptoss_attn_dtype of q,k,v,o,d_o,dq,dk,dv */
+
+    int32_t B, H, G, Sq, Skv, D;
+    int32_t window;         /* 0 = full causal; else sliding window length */
+    int32_t q_offset;       /* absolute position of query row 0 (reference start_q) */
+    float scale;            /* softmax scale (reference sm_scale) */
+    int32_t reserved0;
+
+    const void *q, *k, *v;
+    const float *sinks;     /* optional */
+    const int32_t *seqlens; /* optional */
+    void *o;
+    float *lse;
+
+    const void *d_o;
+    void *dq, *dk, *dv;
+    float *dsinks;          /* optional: NULL skips the sink gradient */
+    float *delta;           /* (B,H,Sq) fp32 scratch written by bwd_preprocess */
+
+    gptoss_attn_strides q_stride, k_stride, v_stride, o_stride;
+    gptoss_attn_strides do_stride, dq_stride, dk_stride, dv_stride;
+} gptoss_attn_params;
+
+/* Library/ABI version (GPTOSS_ATTN_ABI_VERSION it was built with). */
+int gptoss_attn_version(void);
+
+/* Text for a status code returned by any entry point (never NULL). */
+const char *gptoss_attn_status_string(int status);
+
+/*
+ * Forward: O and logsumexp.  Replaces the `_attn_fwd` launch in
+ * `_attention.forward` (attention_kernel.py:11-100, 241-262) including the
+ * output transpose copy at :272 (O is written directly in the caller's layout).
+ * Reads q,k,v,sinks,seqlens; writes o,lse.
+ */
+int gptoss_attn_fwd(const gptoss_attn_params *params, void *stream);
+
+/*
+ * Backward step 1: delta = rowsum(dO * O).  Replaces `_attn_bwd_precompute_D`
+ * (attention_kernel.py:102-120, 304-313) including the dO transpose copy at
+ * :290.  When dsinks != NULL it also produces
+ * dsinks[h] = -sum_{b,i} exp(sinks[h] - lse) * delta   (attention_kernel.py:173-176)
+ * without atomics.  Reads o,d_o,lse,sinks; writes delta,dsinks.
+ */
+int gptoss_attn_bwd_preprocess(const gptoss_attn_params *params, void *stream);
+
+/*
+ * Backward step 2: dK and dV, KV-outer, no atomics (deterministic).  Replaces
+ * the dv/dk halves of `_attn_bwd` (attention_kernel.py:199-212).
+ * Reads q,k,v,d_o,lse,delta,seqlens; writes dk,dv.
+ */
+int gptoss_attn_bwd_dkdv(const gptoss_attn_params *params, void *stream);
+
+/*
+ * Backward step 3: dQ.  Replaces the dq half of `_attn_bwd`
+ * (attention_kernel.py:206-217).  Reads q,k,v,d_o,lse,delta,seqlens; writes dq.
+ */
+int gptoss_attn_bwd_dq(const gptoss_attn_params *params, void *stream);
+
+/*
+ * Whole backward (steps 1-3 on one stream), i.e. `_attention.backward`
+ * (attention_kernel.py:276-344).
+ */
+int gptoss_attn_bwd(const gptoss_attn_params *params, void *stream);
+
+/*
+ * Host-only argument check used by every entry point; `need_bwd` != 0 also
+ * requires the backward tensors.  Callable without a GPU.
+ */
+int gptoss_attn_validate(const gptoss_attn_params *params, int need_bwd);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GPTOSS_ATTN_H */

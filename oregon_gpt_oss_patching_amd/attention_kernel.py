@@ -1,0 +1,200 @@
+"""Drop-in for the reference's `attention_kernel.py`, backed by hand-written
+gfx950 HIP kernels instead of Triton.
+
+Same public names and call conventions as the reference module:
+
+* `attention(q, k, v, sinks, sm_scale, bandwidth, start_q)` -- positional, like
+  `_attention.apply` (attention_kernel.py:220-347).  q is (B, H, S, D), k and v
+  are (B, G, S_kv, D), the result is (B, S, H, D).
+* `triton_flash_attention(module, query, key, value, attention_mask, scaling,
+  dropout=0.0, **kwargs) -> (attn_output, None)` -- the Hugging Face attention
+  interface (attention_kernel.py:348-358).  The name is kept so that
+  `modeling_gpt_oss.eager_attention_forward = triton_flash_attention` keeps
+  working; there is no Triton underneath.
+
+Differences from the reference, none of which change a result it can produce:
+no padding copies of q/k/v (rows are bounds-checked in the kernels), O is written
+directly in (B, S, H, D) and dO read directly from it (no transpose copies,
+attention_kernel.py:272,290), dK/dV/dSinks are produced without atomics and need
+no zero-fill, `sinks=None` works in backward (the reference raises at :344), and
+an optional `seqlens` (right-padding lengths) is accepted.
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import _lib
+
+__all__ = ["attention", "triton_flash_attention", "hip_flash_attention", "attention_forward", "attention_backward"]
+
+_DTYPES = {torch.bfloat16: _lib.DTYPE_BF16}
+
+
+def _strides_bhs(t: torch.Tensor, layout: str):
+    """(b, h, s) element strides of a 4-D tensor given as 'bhsd' or 'bshd'."""
+    st = t.stride()
+    if layout == "bhsd":
+        return st[0], st[1], st[2]
+    return st[0], st[2], st[1]
+
+
+def _row_contiguous(t: torch.Tensor) -> torch.Tensor:
+    """The kernels need unit stride along head_dim and 16-byte aligned rows."""
+    if t.stride(-1) != 1 or any((s * t.element_size()) % 16 for s in t.stride()[:-1]) or t.data_ptr() % 16:
+        return t.contiguous()
+    return t
+
+
+def _set(st, triple):
+    st.b, st.h, st.s = (int(x) for x in triple)
+
+
+def _check_inputs(q, k, v, sinks):
+    if not (q.is_cuda and k.is_cuda and v.is_cuda):
+        raise RuntimeError("gptoss attention runs on the GPU only (HIP kernels); got a CPU tensor")
+    if q.dtype not in _DTYPES or k.dtype != q.dtype or v.dtype != q.dtype:
+        raise RuntimeError(f"unsupported dtypes {q.dtype}/{k.dtype}/{v.dtype}: bfloat16 tensors are required")
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+        raise RuntimeError("q must be (B,H,S,D) and k, v (B,G,S_kv,D)")
+    if k.shape != v.shape or q.shape[0] != k.shape[0] or q.shape[3] != k.shape[3]:
+        raise RuntimeError(f"shape mismatch: q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)}")
+    if sinks is not None and sinks.numel() != q.shape[1]:
+        raise RuntimeError("sinks must hold one logit per query head")
+
+
+def _base_params(q, k, v, sinks32, seqlens, scale, window, q_offset):
+    p = _lib.new_params()
+    b, h, sq, d = q.shape
+    g, skv = k.shape[1], k.shape[2]
+    p.dtype = _DTYPES[q.dtype]
+    p.B, p.H, p.G, p.Sq, p.Skv, p.D = b, h, g, sq, skv, d
+    p.window = int(window or 0)
+    p.q_offset = int(q_offset or 0)
+    p.scale = float(scale)
+    p.q, p.k, p.v = q.data_ptr(), k.data_ptr(), v.data_ptr()
+    p.sinks = sinks32.data_ptr() if sinks32 is not None else None
+    p.seqlens = seqlens.data_ptr() if seqlens is not None else None
+    _set(p.q_stride, _strides_bhs(q, "bhsd"))
+    _set(p.k_stride, _strides_bhs(k, "bhsd"))
+    _set(p.v_stride, _strides_bhs(v, "bhsd"))
+    return p
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _prep_seqlens(seqlens, device, batch):
+    if seqlens is None:
+        return None
+    sl = torch.as_tensor(seqlens, device=device).to(torch.int32).contiguous()
+    if sl.numel() != batch:
+        raise RuntimeError("seqlens must hold one length per batch row")
+    return sl
+
+
+def attention_forward(q, k, v, sinks, sm_scale, window=None, q_offset=0, seqlens=None):
+    """Runs the forward kernel.  Returns (o (B,S,H,D), lse (B,H,S) fp32)."""
+    _check_inputs(q, k, v, sinks)
+    q, k, v = _row_contiguous(q), _row_contiguous(k), _row_contiguous(v)
+    b, h, sq, d = q.shape
+    sinks32 = None if sinks is None else sinks.detach().to(torch.float32).contiguous()
+    sl = _prep_seqlens(seqlens, q.device, b)
+    o = torch.empty((b, sq, h, d), dtype=q.dtype, device=q.device)
+    lse = torch.empty((b, h, sq), dtype=torch.float32, device=q.device)
+    with torch.cuda.device(q.device):
+        p = _base_params(q, k, v, sinks32, sl, sm_scale, window, q_offset)
+        p.o, p.lse = o.data_ptr(), lse.data_ptr()
+        _set(p.o_stride, _strides_bhs(o, "bshd"))
+        _lib.call("gptoss_attn_fwd", p, _stream(q))
+    return o, lse
+
+
+def attention_backward(q, k, v, sinks, o, lse, d_o, sm_scale, window=None, q_offset=0, seqlens=None,
+                       need_dsinks=True):
+    """Runs the three backward kernels.  o and d_o are (B,S,H,D).
+    Returns (dq, dk, dv, dsinks_fp32_or_None)."""
+    _check_inputs(q, k, v, sinks)
+    q, k, v = _row_contiguous(q), _row_contiguous(k), _row_contiguous(v)
+    o, d_o = _row_contiguous(o), _row_contiguous(d_o)
+    b, h, sq, d = q.shape
+    sinks32 = None if sinks is None else sinks.detach().to(torch.float32).contiguous()
+    sl = _prep_seqlens(seqlens, q.device, b)
+    dq = torch.empty((b, h, sq, d), dtype=q.dtype, device=q.device)
+    dk = torch.empty(k.shape, dtype=k.dtype, device=q.device)
+    dv = torch.empty(v.shape, dtype=v.dtype, device=q.device)
+    delta = torch.empty((b, h, sq), dtype=torch.float32, device=q.device)
+    dsinks = torch.empty((h,), dtype=torch.float32, device=q.device) if need_dsinks else None
+    with torch.cuda.device(q.device):
+        p = _base_params(q, k, v, sinks32, sl, sm_scale, window, q_offset)
+        p.o, p.lse = o.data_ptr(), lse.data_ptr()
+        _set(p.o_stride, _strides_bhs(o, "bshd"))
+        p.d_o = d_o.data_ptr()
+        _set(p.do_stride, _strides_bhs(d_o, "bshd"))
+        p.dq, p.dk, p.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
+        _set(p.dq_stride, _strides_bhs(dq, "bhsd"))
+        _set(p.dk_stride, _strides_bhs(dk, "bhsd"))
+        _set(p.dv_stride, _strides_bhs(dv, "bhsd"))
+        p.delta = delta.data_ptr()
+        p.dsinks = dsinks.data_ptr() if dsinks is not None else None
+        _lib.call("gptoss_attn_bwd", p, _stream(q))
+    return dq, dk, dv, dsinks
+
+
+class _attention(torch.autograd.Function):
+    """Same argument list and gradient tuple as the reference's `_attention`
+    (attention_kernel.py:220-344), plus an optional trailing `seqlens`."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, sinks, sm_scale, bandwidth, start_q, seqlens=None):
+        q_offset = 0
+        if start_q is not None:
+            q_offset = int(start_q.item()) if torch.is_tensor(start_q) else int(start_q)
+        o, lse = attention_forward(q, k, v, sinks, sm_scale, bandwidth, q_offset, seqlens)
+        ctx.save_for_backward(q, k, v, sinks, o, lse, seqlens if torch.is_tensor(seqlens) else None)
+        ctx.seqlens_list = None if torch.is_tensor(seqlens) else seqlens
+        ctx.sm_scale = sm_scale
+        ctx.bandwidth = bandwidth
+        ctx.q_offset = q_offset
+        return o
+
+    @staticmethod
+    def backward(ctx, do):
+        q, k, v, sinks, o, lse, seqlens_t = ctx.saved_tensors
+        seqlens = seqlens_t if seqlens_t is not None else ctx.seqlens_list
+        need_ds = sinks is not None and ctx.needs_input_grad[3]
+        dq, dk, dv, dsinks = attention_backward(
+            q, k, v, sinks, o, lse, do, ctx.sm_scale, ctx.bandwidth, ctx.q_offset, seqlens, need_dsinks=need_ds)
+        if dsinks is not None:
+            dsinks = dsinks.to(sinks.dtype).view_as(sinks)
+        return dq, dk, dv, dsinks, None, None, None, None
+
+
+attention = _attention.apply
+
+
+def hip_flash_attention(
+    module,
+    query: torch.Tensor,
+    key: torch.Tensor,
+    value: torch.Tensor,
+    attention_mask: Optional[torch.Tensor],
+    scaling: float,
+    dropout: float = 0.0,
+    **kwargs,
+):
+    """Hugging Face attention-interface adapter (attention_kernel.py:348-358).
+
+    Like the reference it ignores `attention_mask` and `dropout`: causality and the
+    sliding window come from `module.sliding_window`, the sink logits from
+    `module.sinks`.  A caller with right-padded batches may pass `seqlens=` in
+    kwargs."""
+    out = attention(query, key, value, module.sinks, scaling, module.sliding_window, None,
+                    kwargs.get("seqlens"))
+    return out, None
+
+
+# The reference's public name, kept so existing patch code keeps working.
+triton_flash_attention = hip_flash_attention

@@ -1,0 +1,179 @@
+// Forward kernel: O = softmax([S, sink]) V without the sink column, plus the
+// row logsumexp.  Stands in for the reference's `_attn_fwd`
+// (attention_kernel.py:11-100).
+//
+// Work split.  A workgroup is 4 wavefronts.  Each wavefront owns 32 query rows
+// of ONE query head; the 4 wavefronts of a workgroup are HPB query heads of the
+// same KV head times 4/HPB consecutive 32-row slabs, so every K/V tile staged in
+// LDS is shared by the whole GQA group slice.  KV tiles are 64 keys.
+//
+// Per tile the wavefront computes S^T = K Q^T (K rows are the MFMA A operand
+// from LDS, Q^T lives in registers as the B operand), so a lane owns one query
+// row and its 32 logits sit in its own registers: the row max / row sum are
+// in-lane reductions plus one exchange with lane^32.  exp2 is used with
+// scale*log2(e) folded into one FMA.  P^T goes straight from the C registers
+// into the B operand of O^T += V^T P^T; V^T fragments come from the row-major
+// LDS tile through ds_read_b64_tr_b16.
+#pragma once
+#include "attn_common.h"
+
+namespace gptoss {
+
+template <int HPB>
+__global__ __launch_bounds__(256) void attn_fwd_kernel(const KArgs a) {
+    constexpr int QSUB = 4 / HPB;      // 32-row slabs per workgroup
+    constexpr int BM = 32 * QSUB;      // query rows per workgroup
+    __shared__ __attribute__((aligned(16))) bf16 smem[2][2][kTileElems];
+
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int l32 = lane & 31, half = lane >> 5;
+
+    // workgroup -> (kv head, head chunk, batch, query tile); the kv head is the
+    // fastest index so that with G == 8 each XCD (workgroups are dealt round-robin
+    // over the 8 XCDs) keeps one KV head's K/V in its own L2.  Query tiles run from
+    // the last (longest key loop) to the first.
+    const int n_hc = (a.r + HPB - 1) / HPB;
+    int bid = blockIdx.x;
+    const int g = bid % a.G; bid /= a.G;
+    const int hc = bid % n_hc; bid /= n_hc;
+    const int b = bid % a.B; bid /= a.B;
+    const int n_qt = (a.Sq + BM - 1) / BM;
+    const int qt = n_qt - 1 - bid;
+
+    const int hsel = hc * HPB + (w % HPB);
+    const bool active = hsel < a.r;
+    const int head = g * a.r + (active ? hsel : 0);
+    const int qw0 = qt * BM + 32 * (w / HPB);          // first query row of this wavefront
+
+    const int kv_len = a.seqlens ? min(a.Skv, a.seqlens[b]) : a.Skv;
+    const int q_len = a.seqlens ? a.seqlens[b] : 0x7fffffff;
+    const int weff = a.window ? a.window : 0x3fffffff;
+
+    // key range of the workgroup (union over its wavefronts)
+    const int bpos0 = a.q_offset + qt * BM;
+    const int bpos1 = min(a.q_offset + min(a.Sq, (qt + 1) * BM) - 1, q_len - 1);
+    const int hi = bpos1 >= bpos0 ? min(kv_len, bpos1 + 1) : 0;   // no key at all for a fully padded tile
+    const int lo = max(0, bpos0 - weff + 1);
+    const int t_lo = lo / kTile;
+    const int t_hi = hi > 0 ? (hi + kTile - 1) / kTile : 0;
+
+    // this wavefront's own row range (absolute positions)
+    const int wpos0 = a.q_offset + qw0;
+    const int wpos1 = min(a.q_offset + min(a.Sq, qw0 + 32) - 1, q_len - 1);
+    const int p = wpos0 + l32;                          // this lane's query position
+    const bool p_ok = (qw0 + l32 < a.Sq) && (p < q_len);
+
+    const bf16 *kbase = a.k + (int64_t)b * a.ks.b + (int64_t)g * a.ks.h;
+    const bf16 *vbase = a.v + (int64_t)b * a.vs.b + (int64_t)g * a.vs.h;
+
+    // Q^T fragments (B operand), resident for the whole key loop
+    bf16x8 qf[4];
+    {
+        const bf16 *qrow = a.q + (int64_t)b * a.qs.b + (int64_t)head * a.qs.h + (int64_t)(qw0 + l32) * a.qs.s;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            u32x4 z = {0u, 0u, 0u, 0u};
+            if (qw0 + l32 < a.Sq) z = *reinterpret_cast<const u32x4 *>(qrow + 16 * ks + 8 * half);
+            qf[ks] = as_bf16x8(z);
+        }
+    }
+
+    const float c = a.scale_log2;
+    const float sink2 = (a.sinks ? a.sinks[head] : 0.0f) * kLog2e;
+    float m = sink2;       // running max, log2 domain; starts at the sink logit (ref :53)
+    float l = 0.0f;        // this lane's share of the running sum (own keys only)
+    f32x16 o[2];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) { o[0][i] = 0.0f; o[1][i] = 0.0f; }
+
+    TileRegs kr, vr;
+    if (t_lo < t_hi) {
+        tile_load(kr, kbase, a.ks.s, t_lo * kTile, a.Skv, tid);
+        tile_load(vr, vbase, a.vs.s, t_lo * kTile, a.Skv, tid);
+    }
+
+    for (int t = t_lo; t < t_hi; ++t) {
+        const int buf = (t - t_lo) & 1;
+        bf16 *ksm = smem[buf][0], *vsm = smem[buf][1];
+        tile_store(ksm, kr, tid);
+        tile_store(vsm, vr, tid);
+        __syncthreads();
+        if (t + 1 < t_hi) {
+            tile_load(kr, kbase, a.ks.s, (t + 1) * kTile, a.Skv, tid);
+            tile_load(vr, vbase, a.vs.s, (t + 1) * kTile, a.Skv, tid);
+        }
+        const int n0 = t * kTile;
+        // tile classification for this wavefront: skip / interior / needs mask
+        const bool skip = !active || n0 > wpos1 || (n0 + kTile - 1) < (wpos0 - weff + 1) || wpos1 < wpos0;
+        if (skip) continue;
+        const bool interior = (n0 + kTile - 1 <= wpos0) && (n0 > wpos1 - weff) && (n0 + kTile <= kv_len) &&
+                              (a.q_offset + qw0 + 31 <= wpos1);
+
+        f32x16 s[2];
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) s[blk][i] = 0.0f;
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) s[blk] = mfma_bf16(frag_nat(ksm, blk, ks, lane), qf[ks], s[blk]);
+        }
+        if (!interior) {
+#pragma unroll
+            for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int j = n0 + 32 * blk + crow(i, half);
+                    const bool vis = p_ok && (j <= p) && (j > p - weff) && (j < kv_len);
+                    s[blk][i] = vis ? s[blk][i] : -INFINITY;
+                }
+        }
+        float mx = s[0][0];
+#pragma unroll
+        for (int i = 1; i < 16; ++i) mx = fmaxf(mx, s[0][i]);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[1][i]);
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m, mx * c);
+        if (__builtin_amdgcn_ballot_w64(m_new != m) != 0ull) {
+            const float alpha = fast_exp2(m - m_new);
+            l *= alpha;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) { o[0][i] *= alpha; o[1][i] *= alpha; }
+            m = m_new;
+        }
+        float rs = 0.0f;
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const float pe = fast_exp2(fmaf(s[blk][i], c, -m));
+                s[blk][i] = pe;
+                rs += pe;
+            }
+        l += rs;
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const bf16x8 pf = cfrag(s[blk], u);
+#pragma unroll
+                for (int dblk = 0; dblk < 2; ++dblk)
+                    o[dblk] = mfma_bf16(frag_tr(vsm, blk, u, dblk, lane), pf, o[dblk]);
+            }
+    }
+
+    // epilogue: z = l + exp(sink - m); O = acc / z; M = m + log z   (ref :93-98)
+    const float l_tot = l + __shfl_xor(l, 32);
+    const float z = l_tot + fast_exp2(sink2 - m);
+    const float inv = 1.0f / z;
+    __syncthreads();   // every wavefront is done reading the K/V buffers
+    if (active) {
+        bf16 *stage = &smem[0][0][0] + w * 32 * kLS;
+        bf16 *orow0 = a.o + (int64_t)b * a.os.b + (int64_t)head * a.os.h + (int64_t)qw0 * a.os.s;
+        store_rows32(stage, o, inv, orow0, a.os.s, a.Sq - qw0, lane);
+        if (half == 0 && qw0 + l32 < a.Sq)
+            a.lse[((int64_t)b * a.H + head) * a.Sq + qw0 + l32] = (m + fast_log2(z)) * kLn2;
+    }
+}
+
+}  // namespace gptoss

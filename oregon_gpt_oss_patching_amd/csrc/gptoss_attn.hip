@@ -1,0 +1,173 @@
+// C ABI of the gfx950 GPT-OSS attention library (declared in include/gptoss_attn.h):
+// host-side argument validation, launch geometry, and the kernel launches.
+// No torch headers, no allocation, no global mutable state.
+#include <hip/hip_runtime.h>
+
+#include "../../include/gptoss_attn.h"
+#include "attn_bwd.h"
+#include "attn_common.h"
+#include "attn_fwd.h"
+
+using namespace gptoss;
+
+namespace {
+
+bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// A tensor's rows must start on 16-byte boundaries for the 128-bit accesses.
+int check_tensor(const void *p, const gptoss_attn_strides &s, int elem_bytes, int D) {
+    if (!p) return GPTOSS_ATTN_ERR_NULL_TENSOR;
+    if (!aligned16(p)) return GPTOSS_ATTN_ERR_ALIGNMENT;
+    const int64_t per16 = 16 / elem_bytes;
+    if (s.b % per16 || s.h % per16 || s.s % per16) return GPTOSS_ATTN_ERR_ALIGNMENT;
+    if (s.s < D) return GPTOSS_ATTN_ERR_STRIDE;
+    return GPTOSS_ATTN_OK;
+}
+
+Strides cvt(const gptoss_attn_strides &s) { return Strides{s.b, s.h, s.s}; }
+
+KArgs make_args(const gptoss_attn_params *p) {
+    KArgs a{};
+    a.q = static_cast<const bf16 *>(p->q);
+    a.k = static_cast<const bf16 *>(p->k);
+    a.v = static_cast<const bf16 *>(p->v);
+    a.sinks = p->sinks;
+    a.seqlens = p->seqlens;
+    a.o = static_cast<bf16 *>(p->o);
+    a.lse = p->lse;
+    a.d_o = static_cast<const bf16 *>(p->d_o);
+    a.dq = static_cast<bf16 *>(p->dq);
+    a.dk = static_cast<bf16 *>(p->dk);
+    a.dv = static_cast<bf16 *>(p->dv);
+    a.dsinks = p->dsinks;
+    a.delta = p->delta;
+    a.qs = cvt(p->q_stride); a.ks = cvt(p->k_stride); a.vs = cvt(p->v_stride); a.os = cvt(p->o_stride);
+    a.dos = cvt(p->do_stride); a.dqs = cvt(p->dq_stride); a.dks = cvt(p->dk_stride); a.dvs = cvt(p->dv_stride);
+    a.B = p->B; a.H = p->H; a.G = p->G; a.Sq = p->Sq; a.Skv = p->Skv;
+    a.r = p->H / p->G;
+    a.window = p->window;
+    a.q_offset = p->q_offset;
+    a.scale = p->scale;
+    a.scale_log2 = p->scale * kLog2e;
+    return a;
+}
+
+int hpb_for(int r) { return r >= 4 ? 4 : (r >= 2 ? 2 : 1); }
+
+int launch_status() {
+    const hipError_t e = hipGetLastError();
+    return e == hipSuccess ? GPTOSS_ATTN_OK : static_cast<int>(e);
+}
+
+}  // namespace
+
+extern "C" {
+
+int gptoss_attn_version(void) { return GPTOSS_ATTN_ABI_VERSION; }
+
+const char *gptoss_attn_status_string(int status) {
+    switch (status) {
+        case GPTOSS_ATTN_OK: return "ok";
+        case GPTOSS_ATTN_ERR_NULL_PARAMS: return "params pointer is NULL";
+        case GPTOSS_ATTN_ERR_NULL_TENSOR: return "a required tensor pointer is NULL";
+        case GPTOSS_ATTN_ERR_HEAD_DIM: return "head_dim must be 64";
+        case GPTOSS_ATTN_ERR_HEADS: return "H and G must be positive and H divisible by G";
+        case GPTOSS_ATTN_ERR_SHAPE: return "B, Sq, Skv must be positive; window, q_offset non-negative; scale positive and finite";
+        case GPTOSS_ATTN_ERR_DTYPE: return "unsupported dtype";
+        case GPTOSS_ATTN_ERR_ALIGNMENT: return "tensor base or stride is not 16-byte aligned";
+        case GPTOSS_ATTN_ERR_STRIDE: return "sequence stride smaller than head_dim";
+        case GPTOSS_ATTN_ERR_ABI: return "struct_size does not match this library";
+        default: return status > 0 ? "HIP runtime error (status is the hipError_t)" : "unknown status";
+    }
+}
+
+int gptoss_attn_validate(const gptoss_attn_params *p, int need_bwd) {
+    if (!p) return GPTOSS_ATTN_ERR_NULL_PARAMS;
+    if (p->struct_size != sizeof(gptoss_attn_params)) return GPTOSS_ATTN_ERR_ABI;
+    if (p->dtype != GPTOSS_ATTN_BF16) return GPTOSS_ATTN_ERR_DTYPE;
+    if (p->D != kD) return GPTOSS_ATTN_ERR_HEAD_DIM;
+    if (p->H <= 0 || p->G <= 0 || p->H % p->G) return GPTOSS_ATTN_ERR_HEADS;
+    if (p->B <= 0 || p->Sq <= 0 || p->Skv <= 0 || p->window < 0 || p->q_offset < 0) return GPTOSS_ATTN_ERR_SHAPE;
+    if (!(p->scale > 0.0f) || !(p->scale < 3.0e38f)) return GPTOSS_ATTN_ERR_SHAPE;
+    const int eb = 2;
+    int rc;
+    if ((rc = check_tensor(p->q, p->q_stride, eb, p->D))) return rc;
+    if ((rc = check_tensor(p->k, p->k_stride, eb, p->D))) return rc;
+    if ((rc = check_tensor(p->v, p->v_stride, eb, p->D))) return rc;
+    if ((rc = check_tensor(p->o, p->o_stride, eb, p->D))) return rc;
+    if (!p->lse) return GPTOSS_ATTN_ERR_NULL_TENSOR;
+    if (need_bwd) {
+        if ((rc = check_tensor(p->d_o, p->do_stride, eb, p->D))) return rc;
+        if ((rc = check_tensor(p->dq, p->dq_stride, eb, p->D))) return rc;
+        if ((rc = check_tensor(p->dk, p->dk_stride, eb, p->D))) return rc;
+        if ((rc = check_tensor(p->dv, p->dv_stride, eb, p->D))) return rc;
+        if (!p->delta) return GPTOSS_ATTN_ERR_NULL_TENSOR;
+    }
+    return GPTOSS_ATTN_OK;
+}
+
+int gptoss_attn_fwd(const gptoss_attn_params *p, void *stream) {
+    const int rc = gptoss_attn_validate(p, 0);
+    if (rc) return rc;
+    const KArgs a = make_args(p);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int hpb = hpb_for(a.r);
+    const int bm = 32 * (4 / hpb);
+    const int n_hc = (a.r + hpb - 1) / hpb;
+    const unsigned grid = (unsigned)(a.G * n_hc * a.B * ((a.Sq + bm - 1) / bm));
+    if (hpb == 4) hipLaunchKernelGGL(attn_fwd_kernel<4>, dim3(grid), dim3(256), 0, st, a);
+    else if (hpb == 2) hipLaunchKernelGGL(attn_fwd_kernel<2>, dim3(grid), dim3(256), 0, st, a);
+    else hipLaunchKernelGGL(attn_fwd_kernel<1>, dim3(grid), dim3(256), 0, st, a);
+    return launch_status();
+}
+
+int gptoss_attn_bwd_preprocess(const gptoss_attn_params *p, void *stream) {
+    const int rc = gptoss_attn_validate(p, 1);
+    if (rc) return rc;
+    const KArgs a = make_args(p);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int64_t rows = (int64_t)a.B * a.H * a.Sq;
+    hipLaunchKernelGGL(attn_bwd_delta_kernel, dim3((unsigned)((rows + 31) / 32)), dim3(256), 0, st, a);
+    int s = launch_status();
+    if (s) return s;
+    if (a.dsinks) {
+        hipLaunchKernelGGL(attn_bwd_dsinks_kernel, dim3((unsigned)a.H), dim3(256), 0, st, a);
+        s = launch_status();
+    }
+    return s;
+}
+
+int gptoss_attn_bwd_dkdv(const gptoss_attn_params *p, void *stream) {
+    const int rc = gptoss_attn_validate(p, 1);
+    if (rc) return rc;
+    const KArgs a = make_args(p);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const unsigned grid = (unsigned)(a.G * a.B * ((a.Skv + 127) / 128));
+    hipLaunchKernelGGL(attn_bwd_dkdv_kernel, dim3(grid), dim3(256), 0, st, a);
+    return launch_status();
+}
+
+int gptoss_attn_bwd_dq(const gptoss_attn_params *p, void *stream) {
+    const int rc = gptoss_attn_validate(p, 1);
+    if (rc) return rc;
+    const KArgs a = make_args(p);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int hpb = hpb_for(a.r);
+    const int bm = 32 * (4 / hpb);
+    const int n_hc = (a.r + hpb - 1) / hpb;
+    const unsigned grid = (unsigned)(a.G * n_hc * a.B * ((a.Sq + bm - 1) / bm));
+    if (hpb == 4) hipLaunchKernelGGL(attn_bwd_dq_kernel<4>, dim3(grid), dim3(256), 0, st, a);
+    else if (hpb == 2) hipLaunchKernelGGL(attn_bwd_dq_kernel<2>, dim3(grid), dim3(256), 0, st, a);
+    else hipLaunchKernelGGL(attn_bwd_dq_kernel<1>, dim3(grid), dim3(256), 0, st, a);
+    return launch_status();
+}
+
+int gptoss_attn_bwd(const gptoss_attn_params *p, void *stream) {
+    int rc = gptoss_attn_bwd_preprocess(p, stream);
+    if (rc) return rc;
+    rc = gptoss_attn_bwd_dkdv(p, stream);
+    if (rc) return rc;
+    return gptoss_attn_bwd_dq(p, stream);
+}
+
+}  // extern "C"
