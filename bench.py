@@ -1,0 +1,186 @@
+#!/usr/bin/env python3
+"""Benchmark of the attention hot path on one MI355X.
+
+A "step" is one forward + backward of a single GPT-OSS-20B attention layer
+(64 query heads over 8 KV heads, head_dim 64, bf16, B=1) on synthetic N(0,1)
+inputs already resident in HBM.  The headline workload is the full-causal layer
+at S=16384; the same shape with sliding window 128 is timed next to it to report
+the tile-skipping speedup.
+
+Prints ONE JSON line.  `value` is algorithmic TFLOP/s of fwd+bwd
+(FLOPs = 14 * D * pairs * B * H, pairs = S(S+1)/2), `roofline` describes the
+dominant kernel, `cpu_baseline` is the eager fp32 restatement timed on the host
+cores on a bounded sample of the same workload.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2516.6   # MI355X dense bf16 MFMA peak
+PEAK_HBM_GBS = 8000.0
+
+
+def pairs(s, w):
+    return s * (s + 1) // 2 if not w or w >= s else w * s - w * (w - 1) // 2
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--seq", type=int, default=16384)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--cpu-seq", type=int, default=16384, help="sequence length of the CPU-baseline sample")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build measures one GPU only (the attention op has no cross-GPU "
+              "exchange; every box here has one GPU). Run with --gpus 1.", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from oregon_gpt_oss_patching_amd import _lib
+    from oregon_gpt_oss_patching_amd import attention_kernel as ak
+    from oracle import eager_ref as E
+
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    _lib.load()
+    dev = torch.device("cuda:0")
+    B, H, G, D, S = 1, 64, 8, 64, args.seq
+    scale = 0.125
+    q, k, v, sinks, d_out = (t.to(dev) for t in E.make_inputs(3, B, H, G, S, D, torch.bfloat16))
+    # V as the model delivers it: a transposed view of the (B, S, G, D) projection output
+    v = v.transpose(1, 2).contiguous().transpose(1, 2)
+
+    def make_params(window):
+        """Pre-built parameter block + output buffers, so the timed region is only the launches."""
+        o = torch.empty((B, S, H, D), dtype=q.dtype, device=dev)
+        lse = torch.empty((B, H, S), dtype=torch.float32, device=dev)
+        dq, dk, dv = torch.empty_like(q), torch.empty(k.shape, dtype=k.dtype, device=dev), torch.empty(k.shape, dtype=k.dtype, device=dev)
+        delta = torch.empty((B, H, S), dtype=torch.float32, device=dev)
+        dsinks = torch.empty((H,), dtype=torch.float32, device=dev)
+        s32 = sinks.float().contiguous()
+        p = ak._base_params(q, k, v, s32, None, scale, window, 0)
+        p.o, p.lse = o.data_ptr(), lse.data_ptr()
+        ak._set(p.o_stride, ak._strides_bhs(o, "bshd"))
+        p.d_o = d_out.data_ptr()
+        ak._set(p.do_stride, ak._strides_bhs(d_out, "bshd"))
+        p.dq, p.dk, p.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
+        ak._set(p.dq_stride, ak._strides_bhs(dq, "bhsd"))
+        ak._set(p.dk_stride, ak._strides_bhs(dk, "bhsd"))
+        ak._set(p.dv_stride, ak._strides_bhs(dv, "bhsd"))
+        p.delta, p.dsinks = delta.data_ptr(), dsinks.data_ptr()
+        keep = (o, lse, dq, dk, dv, delta, dsinks, s32)
+        return p, keep
+
+    stream = torch.cuda.current_stream(dev)
+    sptr = stream.cuda_stream
+
+    def step(p):
+        _lib.call("gptoss_attn_fwd", p, sptr)
+        _lib.call("gptoss_attn_bwd", p, sptr)
+
+    def time_steps(p, steps, warmup):
+        for _ in range(warmup):
+            step(p)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step(p)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / steps
+
+    def time_kernel(name, p, iters=10):
+        """Average launch duration of one entry point, HIP events on the launch stream."""
+        evs = []
+        for _ in range(iters):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            _lib.call(name, p, sptr)
+            e1.record(stream)
+            evs.append((e0, e1))
+        torch.cuda.synchronize()
+        ts = [a.elapsed_time(b) for a, b in evs]
+        return statistics.mean(ts)
+
+    p_full, keep_full = make_params(0)
+    p_win, keep_win = make_params(128)
+
+    ms_full = time_steps(p_full, args.steps, args.warmup)
+    ms_win = time_steps(p_win, args.steps, args.warmup)
+
+    kern = {}
+    for tag, p in (("full", p_full), ("win128", p_win)):
+        for name in ("gptoss_attn_fwd", "gptoss_attn_bwd_preprocess", "gptoss_attn_bwd_dkdv", "gptoss_attn_bwd_dq"):
+            kern[f"{tag}.{name[12:]}"] = round(time_kernel(name, p), 4)
+
+    unit = 2 * D * pairs(S, 0) * B * H          # one GEMM over the visible pairs
+    fl_total = 7 * unit
+    tflops = fl_total / (ms_full * 1e-3) / 1e12
+    unit_w = 2 * D * pairs(S, 128) * B * H
+    bytes_total = 2 * B * S * D * (2 * H + 2 * G) + 4 * B * H * S + 2 * B * S * D * (4 * H + 4 * G) + 12 * B * H * S
+
+    # dominant kernel: dkdv computes S, dP, dV, dK = 4 of the 7 algorithmic GEMMs
+    dkdv_ms = kern["full.bwd_dkdv"]
+    dkdv_tflops = 4 * unit / (dkdv_ms * 1e-3) / 1e12
+
+    out = {
+        "metric": "attn fwd+bwd TFLOP/s & % bf16 MFMA peak, GPT-OSS-20B shape, S=16K, 1 GPU",
+        "value": round(tflops, 2),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_full, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"GPT-OSS-20B attention layer fwd+bwd, full causal, B=1 S={S} H=64 G=8 D=64",
+                   "window_variant": "same shape, sliding window 128"},
+        "pct_bf16_mfma_peak": round(100.0 * tflops / PEAK_BF16_TFLOPS, 2),
+        "window128": {"ms_per_step": round(ms_win, 4),
+                      "tflops": round(7 * unit_w / (ms_win * 1e-3) / 1e12, 2),
+                      "algorithmic_GBs": round(bytes_total / (ms_win * 1e-3) / 1e9, 1),
+                      "frac_hbm_peak": round(bytes_total / (ms_win * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                      "speedup_vs_full": round(ms_full / ms_win, 2),
+                      "speedup_target": S / 256 * 0.5},
+        "kernel_ms": kern,
+        "roofline": {"bound": "mfma", "kernel": "attn_bwd_dkdv_kernel (full causal)",
+                     "achieved": round(dkdv_tflops, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(dkdv_tflops / PEAK_BF16_TFLOPS, 4), "traffic": None},
+    }
+
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(E, args.cpu_seq, D, scale)
+    print(json.dumps(out))
+
+
+def cpu_baseline(E, s, d, scale):
+    """Eager fp32 restatement (forward + autograd backward) on the host cores, on a
+    bounded sample: two query heads sharing one KV head of the full-causal layer."""
+    import torch
+    cores = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(cores)
+    heads = 2
+    q, k, v, sinks, d_out = E.make_inputs(3, 1, heads, 1, s, d, torch.float32)
+    t0 = time.perf_counter()
+    E.eager_attention_grads(q, k, v, sinks, d_out, scale, None)
+    dt = time.perf_counter() - t0
+    fl = 14 * d * pairs(s, 0) * heads
+    return {"value": round(fl / dt / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"{heads} of 64 query heads (one KV head) of the S={s} full-causal layer, eager fp32 fwd + autograd bwd, "
+                      f"{dt:.1f} s wall; algorithmic FLOPs counted as for the GPU"}
+
+
+if __name__ == "__main__":
+    main()

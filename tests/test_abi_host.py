@@ -1,0 +1,132 @@
+"""Host-only checks of the C ABI: the library loads, exports every symbol the
+header declares, the ctypes mirror matches the header, and argument validation
+returns the documented codes.  No kernel is launched."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from oregon_gpt_oss_patching_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "gptoss_attn.h")
+
+
+def _declared_functions():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(gptoss_attn_[a-z_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported():
+    lib = _lib.load()
+    names = _declared_functions()
+    assert set(names) == set(_lib.EXPORTS), names
+    for n in names:
+        assert getattr(lib, n) is not None
+
+
+def test_version_and_status_strings():
+    lib = _lib.load()
+    assert lib.gptoss_attn_version() == _lib.ABI_VERSION
+    assert _lib.status_string(0) == "ok"
+    assert "64" in _lib.status_string(-3)
+    assert "HIP" in _lib.status_string(719)
+
+
+def test_struct_mirror_matches_header_field_order():
+    text = open(HEADER).read()
+    body = re.search(r"typedef struct gptoss_attn_params \{(.*?)\} gptoss_attn_params;", text, re.S).group(1)
+    body = re.sub(r"/\*.*?\*/", "", body, flags=re.S)
+    names = []
+    for decl in body.split(";"):
+        decl = decl.strip()
+        if not decl:
+            continue
+        for part in decl.split(","):
+            names.append(re.findall(r"[A-Za-z_][A-Za-z_0-9]*", part)[-1])
+    assert names == [f[0] for f in _lib.Params._fields_]
+    assert ctypes.sizeof(_lib.Params) == 344
+
+
+def _valid_params():
+    """A parameter block that passes validation (fake, aligned, never dereferenced)."""
+    p = _lib.new_params()
+    p.dtype = _lib.DTYPE_BF16
+    p.B, p.H, p.G, p.Sq, p.Skv, p.D = 1, 8, 2, 128, 128, 64
+    p.scale = 0.125
+    fake = 0x1000
+    for f in ("q", "k", "v", "o", "lse", "d_o", "dq", "dk", "dv", "delta"):
+        setattr(p, f, fake)
+    for st in ("q_stride", "k_stride", "v_stride", "o_stride", "do_stride", "dq_stride", "dk_stride", "dv_stride"):
+        s = getattr(p, st)
+        s.b, s.h, s.s = 8 * 128 * 64, 128 * 64, 64
+    return p
+
+
+def _validate(p, bwd=1):
+    return _lib.load().gptoss_attn_validate(ctypes.byref(p), bwd)
+
+
+def test_validate_accepts_good_params():
+    assert _validate(_valid_params()) == 0
+
+
+@pytest.mark.parametrize("mutate,code", [
+    (lambda p: setattr(p, "struct_size", 8), -9),
+    (lambda p: setattr(p, "dtype", 7), -6),
+    (lambda p: setattr(p, "D", 128), -3),
+    (lambda p: setattr(p, "G", 3), -4),
+    (lambda p: setattr(p, "H", 0), -4),
+    (lambda p: setattr(p, "Sq", 0), -5),
+    (lambda p: setattr(p, "window", -1), -5),
+    (lambda p: setattr(p, "q_offset", -2), -5),
+    (lambda p: setattr(p, "scale", 0.0), -5),
+    (lambda p: setattr(p, "scale", float("nan")), -5),
+    (lambda p: setattr(p, "q", None), -2),
+    (lambda p: setattr(p, "lse", None), -2),
+    (lambda p: setattr(p, "dv", None), -2),
+    (lambda p: setattr(p, "delta", None), -2),
+    (lambda p: setattr(p, "k", 0x1008), -7),
+    (lambda p: setattr(p.v_stride, "s", 68), -7),
+    (lambda p: setattr(p.v_stride, "s", 32), -8),
+])
+def test_validate_error_codes(mutate, code):
+    p = _valid_params()
+    mutate(p)
+    assert _validate(p) == code
+    assert _lib.status_string(code) not in ("ok", "unknown status")
+
+
+def test_forward_only_validation_ignores_backward_tensors():
+    p = _valid_params()
+    p.dq = None
+    p.delta = None
+    assert _validate(p, 0) == 0 and _validate(p, 1) == -2
+
+
+def test_null_params_pointer():
+    lib = _lib.load()
+    assert lib.gptoss_attn_validate(None, 0) == -1
+    assert lib.gptoss_attn_fwd(None, None) == -1
+    assert lib.gptoss_attn_bwd(None, None) == -1
+
+
+def test_entry_points_reject_bad_arguments_before_launching():
+    """Validation is host-side, so a bad block must come back with its code even
+    where there is no GPU to launch on."""
+    p = _valid_params()
+    p.D = 32
+    lib = _lib.load()
+    for name in ("gptoss_attn_fwd", "gptoss_attn_bwd_preprocess", "gptoss_attn_bwd_dkdv",
+                 "gptoss_attn_bwd_dq", "gptoss_attn_bwd"):
+        assert getattr(lib, name)(ctypes.byref(p), None) == -3
+
+
+def test_call_raises_with_status_text():
+    p = _valid_params()
+    p.G = 5
+    with pytest.raises(_lib.GptossAttnError) as ei:
+        _lib.call("gptoss_attn_fwd", p, 0)
+    assert ei.value.status == -4 and "divisible" in str(ei.value)

@@ -1,0 +1,119 @@
+"""The Python drop-in surface on the GPU: autograd.Function, the Hugging Face
+adapter with tensors laid out as GptOssAttention.forward delivers them, output
+layout, and the patched model path."""
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+from oracle import eager_ref as E
+
+pytestmark = pytest.mark.gpu
+SCALE = 0.125
+DEV = "cuda"
+
+
+def rel_l2(a, b):
+    return float((a.double() - b.double()).norm() / (b.double().norm() + 1e-30))
+
+
+def test_autograd_function_matches_oracle():
+    import oregon_gpt_oss_patching_amd as A
+    for w in (None, 32):
+        q, k, v, sinks, d_out = E.make_inputs(5, 2, 8, 2, 192, 64, torch.bfloat16)
+        ref = E.eager_attention_grads(q.float(), k.float(), v.float(), sinks.float(), d_out.float(), SCALE, w)
+        qd, kd, vd, sd = (t.to(DEV).requires_grad_(True) for t in (q, k, v, sinks))
+        out = A.attention(qd, kd, vd, sd, SCALE, w, None)
+        assert out.shape == (2, 192, 8, 64) and out.is_contiguous()
+        out.backward(d_out.to(DEV))
+        assert sd.grad.dtype == sd.dtype and sd.grad.shape == sd.shape
+        for g, r in zip((out, qd.grad, kd.grad, vd.grad, sd.grad), ref):
+            assert rel_l2(g.detach().float().cpu(), r) < 1e-2
+
+
+def test_hf_adapter_with_model_layouts():
+    """q, k contiguous (B,H,S,D); v a transposed view of (B,S,G,D); sinks a bf16
+    Parameter; attention_mask given but ignored; output (B,S,H,D) contiguous."""
+    import oregon_gpt_oss_patching_amd as A
+    b, h, g, s = 2, 16, 4, 160
+    q, k, v, sinks, d_out = E.make_inputs(6, b, h, g, s, 64, torch.bfloat16)
+    ref = E.eager_attention_grads(q.float(), k.float(), v.float(), sinks.float(), d_out.float(), SCALE, 128)
+    qd, kd = q.to(DEV).requires_grad_(True), k.to(DEV).requires_grad_(True)
+    v_bsgd = v.transpose(1, 2).contiguous().to(DEV).requires_grad_(True)
+    vd = v_bsgd.transpose(1, 2)
+    assert not vd.is_contiguous()
+    module = SimpleNamespace(sinks=torch.nn.Parameter(sinks.to(DEV)), sliding_window=128, training=True)
+    mask = torch.zeros(b, 1, s, s, device=DEV, dtype=torch.bfloat16)
+    out, weights = A.triton_flash_attention(module, qd, kd, vd, mask, SCALE, dropout=0.0, sliding_window=128, s_aux=module.sinks)
+    assert weights is None and out.shape == (b, s, h, 64) and out.is_contiguous()
+    out.reshape(b, s, -1).backward(d_out.to(DEV).reshape(b, s, -1))
+    got = (out, qd.grad, kd.grad, v_bsgd.grad.transpose(1, 2), module.sinks.grad)
+    for gt, r in zip(got, ref):
+        assert rel_l2(gt.detach().float().cpu(), r) < 1e-2
+
+
+def test_frozen_sinks_skip_dsinks():
+    import oregon_gpt_oss_patching_amd as A
+    q, k, v, sinks, d_out = E.make_inputs(7, 1, 8, 2, 64, 64, torch.bfloat16)
+    qd, kd, vd = (t.to(DEV).requires_grad_(True) for t in (q, k, v))
+    sd = sinks.to(DEV)      # requires_grad False, as under LoRA
+    out = A.attention(qd, kd, vd, sd, SCALE, None, None)
+    out.backward(d_out.to(DEV))
+    assert sd.grad is None and qd.grad is not None
+
+
+def test_gradient_checkpoint_recompute_is_stable():
+    import torch.utils.checkpoint as cp
+    import oregon_gpt_oss_patching_amd as A
+    q, k, v, sinks, d_out = E.make_inputs(8, 1, 8, 2, 128, 64, torch.bfloat16)
+    qd, kd, vd, sd = (t.to(DEV).requires_grad_(True) for t in (q, k, v, sinks))
+    out = cp.checkpoint(lambda a, b_, c, s_: A.attention(a, b_, c, s_, SCALE, 32, None), qd, kd, vd, sd, use_reentrant=False)
+    out.backward(d_out.to(DEV))
+    g1 = [t.grad.clone() for t in (qd, kd, vd, sd)]
+    for t in (qd, kd, vd, sd):
+        t.grad = None
+    A.attention(qd, kd, vd, sd, SCALE, 32, None).backward(d_out.to(DEV))
+    for a, t in zip(g1, (qd, kd, vd, sd)):
+        assert torch.equal(a, t.grad)
+
+
+def test_patched_gpt_oss_layer_matches_eager():
+    """patch_flash_attention() swaps the function GptOssAttention calls; a 2-layer
+    GPT-OSS-shaped model (one sliding, one full layer) must give, patched, a loss
+    and gradients at least as close to an fp32 eager run as the unpatched bf16 run is."""
+    from transformers import GptOssConfig, GptOssForCausalLM
+    from oregon_gpt_oss_patching_amd import patching
+    cfg = GptOssConfig(vocab_size=512, hidden_size=256, intermediate_size=256, num_hidden_layers=2,
+                       num_attention_heads=16, num_key_value_heads=4, head_dim=64, num_local_experts=4,
+                       num_experts_per_tok=2, sliding_window=32, max_position_embeddings=512,
+                       layer_types=["sliding_attention", "full_attention"], attn_implementation="eager")
+    torch.manual_seed(0)
+    model = GptOssForCausalLM(cfg).to(DEV, torch.bfloat16)
+    with torch.no_grad():
+        for name, prm in model.named_parameters():
+            if name.endswith("sinks"):
+                prm.copy_(torch.randn_like(prm))
+    ids = torch.randint(0, 512, (2, 200), device=DEV)
+
+    def run(m):
+        m.zero_grad(set_to_none=True)
+        out = m(input_ids=ids, labels=ids)
+        out.loss.backward()
+        grads = {n: p.grad.detach().float().clone() for n, p in m.named_parameters() if p.grad is not None}
+        return float(out.loss.detach()), grads
+
+    # ground truth: the same weights in fp32 through the unpatched eager path
+    import copy
+    loss_t, g_t = run(copy.deepcopy(model).float())
+    loss_e, g_e = run(model)                      # bf16 eager (softmax in bf16)
+    patching.patch_flash_attention()
+    try:
+        loss_p, g_p = run(model)                  # bf16 with the HIP kernels
+    finally:
+        patching.unpatch_flash_attention()
+    assert abs(loss_p - loss_t) < 2e-2 * max(1.0, abs(loss_t)), (loss_t, loss_e, loss_p)
+    # the patched gradients must be as close to the fp32 truth as bf16 eager is
+    for n in g_t:
+        if g_t[n].norm() > 1e-6:
+            err_e, err_p = rel_l2(g_e[n], g_t[n]), rel_l2(g_p[n], g_t[n])
+            assert err_p < max(1.5 * err_e, 3e-2), (n, err_p, err_e)

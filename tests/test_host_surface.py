@@ -1,0 +1,51 @@
+"""Host-side checks of the Python surface that mirrors the reference
+(attention_kernel.py:347-358, patching.py:1-10): names, signatures, patching,
+and loud failure on CPU tensors (there is no CPU fallback path)."""
+import inspect
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+import oregon_gpt_oss_patching_amd as A
+from oregon_gpt_oss_patching_amd import attention_kernel as ak
+
+
+def test_public_names_match_reference():
+    assert callable(ak.attention) and callable(ak.triton_flash_attention)
+    sig = inspect.signature(ak.triton_flash_attention)
+    assert list(sig.parameters) == ["module", "query", "key", "value", "attention_mask", "scaling", "dropout", "kwargs"]
+    assert sig.parameters["dropout"].default == 0.0
+
+
+def test_patch_and_unpatch_swap_the_module_global():
+    from transformers.models.gpt_oss import modeling_gpt_oss
+    from oregon_gpt_oss_patching_amd import patching
+    original = modeling_gpt_oss.eager_attention_forward
+    assert patching._original_eager_attention_forward is original
+    patching.patch_flash_attention()
+    try:
+        assert modeling_gpt_oss.eager_attention_forward is ak.triton_flash_attention
+    finally:
+        patching.unpatch_flash_attention()
+    assert modeling_gpt_oss.eager_attention_forward is original
+
+
+def test_cpu_tensors_fail_loudly():
+    q = torch.zeros(1, 8, 16, 64, dtype=torch.bfloat16)
+    k = torch.zeros(1, 2, 16, 64, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        ak.attention(q, k, k, torch.zeros(8), 0.125, None, None)
+    mod = SimpleNamespace(sinks=torch.zeros(8), sliding_window=None)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        A.triton_flash_attention(mod, q, k, k, None, 0.125)
+
+
+def test_stride_helper_layouts():
+    t = torch.empty(2, 5, 3, 64)              # (B, S, H, D)
+    assert ak._strides_bhs(t, "bshd") == (5 * 3 * 64, 64, 3 * 64)
+    u = torch.empty(2, 3, 5, 64)              # (B, H, S, D)
+    assert ak._strides_bhs(u, "bhsd") == (3 * 5 * 64, 5 * 64, 64)
+    v = t.transpose(1, 2)                     # HF's value_states view: (B, H, S, D) strides of (B,S,H,D)
+    assert ak._strides_bhs(v, "bhsd") == (5 * 3 * 64, 64, 3 * 64)
+    assert ak._row_contiguous(v.to(torch.bfloat16)) is not None
