@@ -10,6 +10,13 @@
 #pragma once
 #include "attn_common.h"
 
+// Scheduling fence between software-pipeline phases (keeps early-issued LDS reads early).
+#ifdef GPTOSS_FENCE
+#define GPTOSS_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
+#else
+#define GPTOSS_SCHED_FENCE()
+#endif
+
 namespace gptoss {
 
 // ---------------------------------------------------------------------------------
@@ -59,16 +66,104 @@ __global__ __launch_bounds__(256) void attn_bwd_dsinks_kernel(const KArgs a) {
 }
 
 // ---------------------------------------------------------------------------------
-// dK, dV.  Workgroup = 4 wavefronts x 32 keys = 128 keys of KV head g, batch b.
-// K and V rows of a wavefront stay in registers as MFMA B operands.  The loop
-// streams 64-row Q and dO tiles (plus their lse / delta) of each of the r query
-// heads through LDS:
+// dK, dV.  Workgroup = NW wavefronts x 64 keys of KV head g, batch b.  The K and V
+// rows of a wavefront stay in registers as MFMA B operands (two 32-key blocks, so
+// every Q / dO fragment fetched from LDS feeds two MFMAs).  The loop streams
+// 64-row Q and dO tiles (plus their lse / delta) of each of the r query heads
+// through LDS:
 //   S  = Q K^T, dP = dO V^T         (A = Q / dO rows from LDS, natural reads)
 //   P  = exp2(S*c - lse*log2e),  dS = P * (dP - delta)
 //   dV^T += dO^T P,  dK^T += Q^T dS (A = transposed LDS reads, B = C registers)
-// A lane owns one key; accumulators are written once at the end.
-__global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const KArgs a) {
-    constexpr int BN = 128;
+// A lane owns two keys; accumulators are written once at the end.
+// One 64-row query tile against a wavefront's 64 keys (see attn_bwd_dkdv_kernel).
+// MASKED = false is the interior fast path: every (query, key) pair is visible.
+// In the masked variant `dbase[nb]` is (first query position of the tile) - (this
+// lane's key), or a huge negative number for a dead key, so that pair (row r, key)
+// is visible iff 0 <= dbase + r < weff, tested with one unsigned compare; rows at
+// or beyond `row_lim` (relative to the tile) do not exist.
+template <bool MASKED, int NB>
+__device__ __forceinline__ void dkdv_tile(const bf16 *qsm, const bf16 *gsm, const float *lse_s, const float *del_s,
+                                          const bf16x8 (&kf)[NB][4], const bf16x8 (&vf)[NB][4],
+                                          f32x16 (&dk)[NB][2], f32x16 (&dv)[NB][2], float c, int lane,
+                                          const int (&dbase)[NB], unsigned weff, int row_lim) {
+    const int half = lane >> 5;
+    // LDS reads are issued one phase ahead of the MFMAs that consume them, so the
+    // matrix pipe never waits on an LDS round trip:
+    //   [A frags of block qb] -> S/dP MFMAs -> [transposed frags + row stats] ->
+    //   exp / dS on the VALU (A frags of block qb+1 in flight) -> dV/dK MFMAs.
+    bf16x8 aq[4], ag[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) { aq[ks] = frag_nat(qsm, 0, ks, lane); ag[ks] = frag_nat(gsm, 0, ks, lane); }
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
+        f32x16 s[NB], dp[NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) { s[nb][i] = 0.0f; dp[nb][i] = 0.0f; }
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                s[nb] = mfma_bf16(aq[ks], kf[nb][ks], s[nb]);
+                dp[nb] = mfma_bf16(ag[ks], vf[nb][ks], dp[nb]);
+            }
+        GPTOSS_SCHED_FENCE();
+        bf16x8 agt[2][2], aqt[2][2];
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int dblk = 0; dblk < 2; ++dblk) {
+                agt[u][dblk] = frag_tr(gsm, qb, u, dblk, lane);
+                aqt[u][dblk] = frag_tr(qsm, qb, u, dblk, lane);
+            }
+        f32x4 lv[4], dl[4];
+#pragma unroll
+        for (int a4 = 0; a4 < 4; ++a4) {
+            lv[a4] = *reinterpret_cast<const f32x4 *>(lse_s + 32 * qb + 8 * a4 + 4 * half);
+            dl[a4] = *reinterpret_cast<const f32x4 *>(del_s + 32 * qb + 8 * a4 + 4 * half);
+        }
+        if (qb == 0) {
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) { aq[ks] = frag_nat(qsm, 1, ks, lane); ag[ks] = frag_nat(gsm, 1, ks, lane); }
+        }
+        GPTOSS_SCHED_FENCE();
+#pragma unroll
+        for (int a4 = 0; a4 < 4; ++a4)
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int i = 4 * a4 + e;
+                    float pe = fast_exp2(fmaf(s[nb][i], c, -lv[a4][e]));
+                    if (MASKED) {
+                        const int r = 32 * qb + 8 * a4 + 4 * half + e;
+                        const bool vis = ((unsigned)(dbase[nb] + r) < weff) & (r < row_lim);
+                        pe = vis ? pe : 0.0f;
+                    }
+                    s[nb][i] = pe;
+                    dp[nb][i] = pe * (dp[nb][i] - dl[a4][e]);
+                }
+        GPTOSS_SCHED_FENCE();
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                const bf16x8 pf = cfrag(s[nb], u), dsf = cfrag(dp[nb], u);
+#pragma unroll
+                for (int dblk = 0; dblk < 2; ++dblk) {
+                    dv[nb][dblk] = mfma_bf16(agt[u][dblk], pf, dv[nb][dblk]);
+                    dk[nb][dblk] = mfma_bf16(aqt[u][dblk], dsf, dk[nb][dblk]);
+                }
+            }
+    }
+}
+
+template <int NW, int NB>             // NB = 32-key blocks per wavefront
+__global__ __launch_bounds__(NW * 64, (NB == 1 ? 2 : 1)) void attn_bwd_dkdv_kernel(const KArgs a) {
+    constexpr int NT = NW * 64;
+    constexpr int WK = 32 * NB;        // keys per wavefront
+    constexpr int BN = WK * NW;        // keys per workgroup
     __shared__ __attribute__((aligned(16))) bf16 smem[2][2][kTileElems];
     __shared__ __attribute__((aligned(16))) float sstat[2][2][kTile];
 
@@ -80,8 +175,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const KArgs a) {
     const int b = bid % a.B; bid /= a.B;
     const int kt = bid;                                   // ascending: most work first
     const int j0 = kt * BN;                               // first key of the workgroup
-    const int wj0 = j0 + 32 * w;                          // first key of the wavefront
-    const int jme = wj0 + l32;                            // this lane's key
+    const int wj0 = j0 + WK * w;                          // first key of the wavefront
 
     const int kv_len = a.seqlens ? min(a.Skv, a.seqlens[b]) : a.Skv;
     const int q_len = a.seqlens ? a.seqlens[b] : 0x7fffffff;
@@ -89,7 +183,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const KArgs a) {
 
     // query rows that can see any key of the workgroup
     const int j1 = min(j0 + BN, kv_len) - 1;              // last live key
-    int i_lo = max(0, j0 - a.q_offset);
+    const int i_lo = max(0, j0 - a.q_offset);
     int64_t i_hi64 = min((int64_t)a.Sq, (int64_t)q_len - a.q_offset);
     i_hi64 = min(i_hi64, (int64_t)j1 + weff - a.q_offset);
     const int i_hi = (j1 >= j0) ? (int)max((int64_t)0, i_hi64) : 0;
@@ -99,35 +193,42 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const KArgs a) {
     const int n_it = nq * a.r;
 
     // K, V fragments (B operands): lane = key, slots = head_dim
-    bf16x8 kf[4], vf[4];
-    {
-        const bf16 *krow = a.k + (int64_t)b * a.ks.b + (int64_t)g * a.ks.h + (int64_t)jme * a.ks.s;
-        const bf16 *vrow = a.v + (int64_t)b * a.vs.b + (int64_t)g * a.vs.h + (int64_t)jme * a.vs.s;
+    bf16x8 kf[NB][4], vf[NB][4];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        const int j = wj0 + 32 * nb + l32;
+        const bf16 *krow = a.k + (int64_t)b * a.ks.b + (int64_t)g * a.ks.h + (int64_t)j * a.ks.s;
+        const bf16 *vrow = a.v + (int64_t)b * a.vs.b + (int64_t)g * a.vs.h + (int64_t)j * a.vs.s;
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
             u32x4 zk = {0u, 0u, 0u, 0u}, zv = {0u, 0u, 0u, 0u};
-            if (jme < a.Skv) {
+            if (j < a.Skv) {
                 zk = *reinterpret_cast<const u32x4 *>(krow + 16 * ks + 8 * half);
                 zv = *reinterpret_cast<const u32x4 *>(vrow + 16 * ks + 8 * half);
             }
-            kf[ks] = as_bf16x8(zk);
-            vf[ks] = as_bf16x8(zv);
+            kf[nb][ks] = as_bf16x8(zk);
+            vf[nb][ks] = as_bf16x8(zv);
         }
     }
 
-    f32x16 dk[2], dv[2];
+    f32x16 dk[NB][2], dv[NB][2];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) { dk[0][i] = dk[1][i] = 0.0f; dv[0][i] = dv[1][i] = 0.0f; }
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) { dk[nb][0][i] = dk[nb][1][i] = 0.0f; dv[nb][0][i] = dv[nb][1][i] = 0.0f; }
 
     const float c = a.scale_log2;
-    TileRegs qr, gr;
+    int dead[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) dead[nb] = 0;
+    TileRegs<NT> qr, gr;
     float st = 0.0f;     // lse*log2e (threads 0..63) or delta (threads 64..127) of the staged tile
 
     auto prefetch = [&](int it) {
         const int hq = g * a.r + it / nq;
         const int i0 = (qt_lo + it % nq) * kTile;
-        tile_load(qr, a.q + (int64_t)b * a.qs.b + (int64_t)hq * a.qs.h, a.qs.s, i0, a.Sq, tid);
-        tile_load(gr, a.d_o + (int64_t)b * a.dos.b + (int64_t)hq * a.dos.h, a.dos.s, i0, a.Sq, tid);
+        tile_load<NT>(qr, a.q + (int64_t)b * a.qs.b + (int64_t)hq * a.qs.h, a.qs.s, i0, a.Sq, tid);
+        tile_load<NT>(gr, a.d_o + (int64_t)b * a.dos.b + (int64_t)hq * a.dos.h, a.dos.s, i0, a.Sq, tid);
         if (tid < 128) {
             const int i = i0 + (tid & 63);
             const int64_t off = ((int64_t)b * a.H + hq) * a.Sq + i;
@@ -140,8 +241,8 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const KArgs a) {
     for (int it = 0; it < n_it; ++it) {
         const int buf = it & 1;
         bf16 *qsm = smem[buf][0], *gsm = smem[buf][1];
-        tile_store(qsm, qr, tid);
-        tile_store(gsm, gr, tid);
+        tile_store<NT>(qsm, qr, tid);
+        tile_store<NT>(gsm, gr, tid);
         if (tid < 128) sstat[buf][tid >> 6][tid & 63] = st;
         __syncthreads();
         if (it + 1 < n_it) prefetch(it + 1);
@@ -149,72 +250,104 @@ __global__ __launch_bounds__(256) void attn_bwd_dkdv_kernel(const KArgs a) {
         const int i0 = (qt_lo + it % nq) * kTile;
         const int pos0 = a.q_offset + i0;                                    // first query position of the tile
         const int pos1 = min(a.q_offset + min(a.Sq, i0 + kTile) - 1, q_len - 1);   // last live one
-        const int wj1 = min(wj0 + 32, kv_len) - 1;                           // wavefront's last live key
+        const int wj1 = min(wj0 + WK, kv_len) - 1;                           // wavefront's last live key
         const bool skip = wj1 < wj0 || pos1 < wj0 || pos0 > wj1 + weff - 1 || pos1 < pos0;
         if (skip) continue;
-        const bool interior = (wj0 + 31 <= pos0) && (wj0 > pos1 - weff) && (wj0 + 32 <= kv_len) &&
+        const bool interior = (wj0 + WK - 1 <= pos0) && (wj0 > pos1 - weff) && (wj0 + WK <= kv_len) &&
                               (a.q_offset + i0 + kTile - 1 <= pos1);
         const float *lse_s = sstat[buf][0], *del_s = sstat[buf][1];
-
+        if (interior) {
+            dkdv_tile<false, NB>(qsm, gsm, lse_s, del_s, kf, vf, dk, dv, c, lane, dead, 0u, 0);
+        } else {
+            int dbase[NB];
 #pragma unroll
-        for (int qb = 0; qb < 2; ++qb) {
-            f32x16 s, dp;
-#pragma unroll
-            for (int i = 0; i < 16; ++i) { s[i] = 0.0f; dp[i] = 0.0f; }
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks) {
-                s = mfma_bf16(frag_nat(qsm, qb, ks, lane), kf[ks], s);
-                dp = mfma_bf16(frag_nat(gsm, qb, ks, lane), vf[ks], dp);
+            for (int nb = 0; nb < NB; ++nb) {
+                const int j = wj0 + 32 * nb + l32;
+                dbase[nb] = (j < kv_len) ? pos0 - j : -0x40000000;
             }
-#pragma unroll
-            for (int a4 = 0; a4 < 4; ++a4) {
-                const f32x4 lv = *reinterpret_cast<const f32x4 *>(lse_s + 32 * qb + 8 * a4 + 4 * half);
-                const f32x4 dl = *reinterpret_cast<const f32x4 *>(del_s + 32 * qb + 8 * a4 + 4 * half);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int i = 4 * a4 + e;
-                    float pe = fast_exp2(fmaf(s[i], c, -lv[e]));
-                    if (!interior) {
-                        const int irow = i0 + 32 * qb + 8 * a4 + 4 * half + e;
-                        const int p = a.q_offset + irow;
-                        const bool vis = (irow < a.Sq) && (p < q_len) && (jme <= p) && (jme > p - weff) && (jme < kv_len);
-                        pe = vis ? pe : 0.0f;
-                    }
-                    s[i] = pe;
-                    dp[i] = pe * (dp[i] - dl[e]);
-                }
-            }
-#pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                const bf16x8 pf = cfrag(s, u), dsf = cfrag(dp, u);
-#pragma unroll
-                for (int dblk = 0; dblk < 2; ++dblk) {
-                    dv[dblk] = mfma_bf16(frag_tr(gsm, qb, u, dblk, lane), pf, dv[dblk]);
-                    dk[dblk] = mfma_bf16(frag_tr(qsm, qb, u, dblk, lane), dsf, dk[dblk]);
-                }
-            }
+            const int row_lim = (int)min((int64_t)kTile, min((int64_t)a.Sq, (int64_t)q_len - a.q_offset) - i0);
+            dkdv_tile<true, NB>(qsm, gsm, lse_s, del_s, kf, vf, dk, dv, c, lane, dbase, (unsigned)weff, row_lim);
         }
     }
 
     __syncthreads();
     bf16 *stage = &smem[0][0][0] + w * 32 * kLS;
-    const int nvalid = a.Skv - wj0;
-    store_rows32(stage, dk, a.scale, a.dk + (int64_t)b * a.dks.b + (int64_t)g * a.dks.h + (int64_t)wj0 * a.dks.s,
-                 a.dks.s, nvalid, lane);
-    __builtin_amdgcn_wave_barrier();
-    store_rows32(stage, dv, 1.0f, a.dv + (int64_t)b * a.dvs.b + (int64_t)g * a.dvs.h + (int64_t)wj0 * a.dvs.s,
-                 a.dvs.s, nvalid, lane);
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        const int r0 = wj0 + 32 * nb;
+        const int nvalid = a.Skv - r0;
+        store_rows32(stage, dk[nb], a.scale, a.dk + (int64_t)b * a.dks.b + (int64_t)g * a.dks.h + (int64_t)r0 * a.dks.s,
+                     a.dks.s, nvalid, lane);
+        __builtin_amdgcn_wave_barrier();
+        store_rows32(stage, dv[nb], 1.0f, a.dv + (int64_t)b * a.dvs.b + (int64_t)g * a.dvs.h + (int64_t)r0 * a.dvs.s,
+                     a.dvs.s, nvalid, lane);
+        __builtin_amdgcn_wave_barrier();
+    }
 }
 
 // ---------------------------------------------------------------------------------
-// dQ.  Same decomposition as the forward kernel (wavefront = 32 query rows of one
-// head, K/V tiles shared through LDS by HPB heads of the group):
+// dQ.  Same decomposition as the forward kernel (wavefront = 32*NQB query rows of
+// one head, K/V tiles shared through LDS by HPB heads of the group):
 //   S^T = K Q^T, dP^T = V dO^T, P = exp2(S*c - lse*log2e), dS = P (dP - delta),
 //   dQ^T += K^T dS^T   (A = transposed read of the K tile, B = C registers).
-template <int HPB>
-__global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const KArgs a) {
+template <bool MASKED, int NQB>
+__device__ __forceinline__ void dq_tile(const bf16 *ksm, const bf16 *vsm, const bf16x8 (&qf)[NQB][4],
+                                        const bf16x8 (&gf)[NQB][4], f32x16 (&dq)[NQB][2], const float (&lse2)[NQB],
+                                        const float (&dlt)[NQB], float c, int lane, const int (&dbase)[NQB],
+                                        unsigned weff, int key_lim) {
+    const int half = lane >> 5;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+        f32x16 s[NQB], dp[NQB];
+#pragma unroll
+        for (int qb = 0; qb < NQB; ++qb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) { s[qb][i] = 0.0f; dp[qb][i] = 0.0f; }
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            const bf16x8 ak = frag_nat(ksm, kb, ks, lane);
+            const bf16x8 av = frag_nat(vsm, kb, ks, lane);
+#pragma unroll
+            for (int qb = 0; qb < NQB; ++qb) {
+                s[qb] = mfma_bf16(ak, qf[qb][ks], s[qb]);
+                dp[qb] = mfma_bf16(av, gf[qb][ks], dp[qb]);
+            }
+        }
+#pragma unroll
+        for (int qb = 0; qb < NQB; ++qb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                float pe = fast_exp2(fmaf(s[qb][i], c, -lse2[qb]));
+                if (MASKED) {
+                    const int r = 32 * kb + crow(i, half);
+                    const bool vis = ((unsigned)(dbase[qb] - r) < weff) & (r < key_lim);
+                    pe = vis ? pe : 0.0f;
+                }
+                dp[qb][i] = pe * (dp[qb][i] - dlt[qb]);
+            }
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            bf16x8 akt[2];
+#pragma unroll
+            for (int dblk = 0; dblk < 2; ++dblk) akt[dblk] = frag_tr(ksm, kb, u, dblk, lane);
+#pragma unroll
+            for (int qb = 0; qb < NQB; ++qb) {
+                const bf16x8 dsf = cfrag(dp[qb], u);
+#pragma unroll
+                for (int dblk = 0; dblk < 2; ++dblk) dq[qb][dblk] = mfma_bf16(akt[dblk], dsf, dq[qb][dblk]);
+            }
+        }
+    }
+}
+
+#ifndef GPTOSS_DQ_WAVES
+#define GPTOSS_DQ_WAVES 3
+#endif
+template <int HPB, int NQB>
+__global__ __launch_bounds__(256, GPTOSS_DQ_WAVES) void attn_bwd_dq_kernel(const KArgs a) {
     constexpr int QSUB = 4 / HPB;
-    constexpr int BM = 32 * QSUB;
+    constexpr int WM = 32 * NQB;
+    constexpr int BM = WM * QSUB;
     __shared__ __attribute__((aligned(16))) bf16 smem[2][2][kTileElems];
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
@@ -231,7 +364,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const KArgs a) {
     const int hsel = hc * HPB + (w % HPB);
     const bool active = hsel < a.r;
     const int head = g * a.r + (active ? hsel : 0);
-    const int qw0 = qt * BM + 32 * (w / HPB);
+    const int qw0 = qt * BM + WM * (w / HPB);
 
     const int kv_len = a.seqlens ? min(a.Skv, a.seqlens[b]) : a.Skv;
     const int q_len = a.seqlens ? a.seqlens[b] : 0x7fffffff;
@@ -245,18 +378,20 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const KArgs a) {
     const int t_hi = hi > 0 ? (hi + kTile - 1) / kTile : 0;
 
     const int wpos0 = a.q_offset + qw0;
-    const int wpos1 = min(a.q_offset + min(a.Sq, qw0 + 32) - 1, q_len - 1);
-    const int p = wpos0 + l32;
-    const bool row_ok = qw0 + l32 < a.Sq;
-    const bool p_ok = row_ok && (p < q_len);
+    const int wpos1 = min(a.q_offset + min(a.Sq, qw0 + WM) - 1, q_len - 1);
 
     const bf16 *kbase = a.k + (int64_t)b * a.ks.b + (int64_t)g * a.ks.h;
     const bf16 *vbase = a.v + (int64_t)b * a.vs.b + (int64_t)g * a.vs.h;
 
-    bf16x8 qf[4], gf[4];
-    {
-        const bf16 *qrow = a.q + (int64_t)b * a.qs.b + (int64_t)head * a.qs.h + (int64_t)(qw0 + l32) * a.qs.s;
-        const bf16 *grow = a.d_o + (int64_t)b * a.dos.b + (int64_t)head * a.dos.h + (int64_t)(qw0 + l32) * a.dos.s;
+    bf16x8 qf[NQB][4], gf[NQB][4];
+    float lse2[NQB], dlt[NQB];
+    int pq[NQB];
+#pragma unroll
+    for (int qb = 0; qb < NQB; ++qb) {
+        const int row = qw0 + 32 * qb + l32;
+        const bool row_ok = row < a.Sq;
+        const bf16 *qrow = a.q + (int64_t)b * a.qs.b + (int64_t)head * a.qs.h + (int64_t)row * a.qs.s;
+        const bf16 *grow = a.d_o + (int64_t)b * a.dos.b + (int64_t)head * a.dos.h + (int64_t)row * a.dos.s;
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
             u32x4 zq = {0u, 0u, 0u, 0u}, zg = {0u, 0u, 0u, 0u};
@@ -264,76 +399,66 @@ __global__ __launch_bounds__(256) void attn_bwd_dq_kernel(const KArgs a) {
                 zq = *reinterpret_cast<const u32x4 *>(qrow + 16 * ks + 8 * half);
                 zg = *reinterpret_cast<const u32x4 *>(grow + 16 * ks + 8 * half);
             }
-            qf[ks] = as_bf16x8(zq);
-            gf[ks] = as_bf16x8(zg);
+            qf[qb][ks] = as_bf16x8(zq);
+            gf[qb][ks] = as_bf16x8(zg);
         }
-    }
-    float lse2 = 0.0f, dlt = 0.0f;
-    if (row_ok) {
-        const int64_t off = ((int64_t)b * a.H + head) * a.Sq + qw0 + l32;
-        lse2 = a.lse[off] * kLog2e;
-        dlt = a.delta[off];
+        lse2[qb] = 0.0f;
+        dlt[qb] = 0.0f;
+        if (row_ok) {
+            const int64_t off = ((int64_t)b * a.H + head) * a.Sq + row;
+            lse2[qb] = a.lse[off] * kLog2e;
+            dlt[qb] = a.delta[off];
+        }
+        const int p = a.q_offset + row;
+        pq[qb] = (row_ok && p < q_len) ? p : -0x40000000;
     }
 
     const float c = a.scale_log2;
-    f32x16 dq[2];
+    f32x16 dq[NQB][2];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) { dq[0][i] = 0.0f; dq[1][i] = 0.0f; }
+    for (int qb = 0; qb < NQB; ++qb)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) { dq[qb][0][i] = 0.0f; dq[qb][1][i] = 0.0f; }
 
-    TileRegs kr, vr;
+    TileRegs<256> kr, vr;
     if (t_lo < t_hi) {
-        tile_load(kr, kbase, a.ks.s, t_lo * kTile, a.Skv, tid);
-        tile_load(vr, vbase, a.vs.s, t_lo * kTile, a.Skv, tid);
+        tile_load<256>(kr, kbase, a.ks.s, t_lo * kTile, a.Skv, tid);
+        tile_load<256>(vr, vbase, a.vs.s, t_lo * kTile, a.Skv, tid);
     }
     for (int t = t_lo; t < t_hi; ++t) {
         const int buf = (t - t_lo) & 1;
         bf16 *ksm = smem[buf][0], *vsm = smem[buf][1];
-        tile_store(ksm, kr, tid);
-        tile_store(vsm, vr, tid);
+        tile_store<256>(ksm, kr, tid);
+        tile_store<256>(vsm, vr, tid);
         __syncthreads();
         if (t + 1 < t_hi) {
-            tile_load(kr, kbase, a.ks.s, (t + 1) * kTile, a.Skv, tid);
-            tile_load(vr, vbase, a.vs.s, (t + 1) * kTile, a.Skv, tid);
+            tile_load<256>(kr, kbase, a.ks.s, (t + 1) * kTile, a.Skv, tid);
+            tile_load<256>(vr, vbase, a.vs.s, (t + 1) * kTile, a.Skv, tid);
         }
         const int n0 = t * kTile;
         const bool skip = !active || n0 > wpos1 || (n0 + kTile - 1) < (wpos0 - weff + 1) || wpos1 < wpos0;
         if (skip) continue;
         const bool interior = (n0 + kTile - 1 <= wpos0) && (n0 > wpos1 - weff) && (n0 + kTile <= kv_len) &&
-                              (a.q_offset + qw0 + 31 <= wpos1);
+                              (a.q_offset + qw0 + WM - 1 <= wpos1);
+        if (interior) {
+            dq_tile<false, NQB>(ksm, vsm, qf, gf, dq, lse2, dlt, c, lane, pq, 0u, 0);
+        } else {
+            int dbase[NQB];
 #pragma unroll
-        for (int blk = 0; blk < 2; ++blk) {
-            f32x16 s, dp;
-#pragma unroll
-            for (int i = 0; i < 16; ++i) { s[i] = 0.0f; dp[i] = 0.0f; }
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks) {
-                s = mfma_bf16(frag_nat(ksm, blk, ks, lane), qf[ks], s);
-                dp = mfma_bf16(frag_nat(vsm, blk, ks, lane), gf[ks], dp);
-            }
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                float pe = fast_exp2(fmaf(s[i], c, -lse2));
-                if (!interior) {
-                    const int j = n0 + 32 * blk + crow(i, half);
-                    const bool vis = p_ok && (j <= p) && (j > p - weff) && (j < kv_len);
-                    pe = vis ? pe : 0.0f;
-                }
-                dp[i] = pe * (dp[i] - dlt);
-            }
-#pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                const bf16x8 dsf = cfrag(dp, u);
-#pragma unroll
-                for (int dblk = 0; dblk < 2; ++dblk)
-                    dq[dblk] = mfma_bf16(frag_tr(ksm, blk, u, dblk, lane), dsf, dq[dblk]);
-            }
+            for (int qb = 0; qb < NQB; ++qb) dbase[qb] = pq[qb] - n0;
+            dq_tile<true, NQB>(ksm, vsm, qf, gf, dq, lse2, dlt, c, lane, dbase, (unsigned)weff, kv_len - n0);
         }
     }
     __syncthreads();
     if (active) {
         bf16 *stage = &smem[0][0][0] + w * 32 * kLS;
-        bf16 *row0 = a.dq + (int64_t)b * a.dqs.b + (int64_t)head * a.dqs.h + (int64_t)qw0 * a.dqs.s;
-        store_rows32(stage, dq, a.scale, row0, a.dqs.s, a.Sq - qw0, lane);
+#pragma unroll
+        for (int qb = 0; qb < NQB; ++qb) {
+            const int r0 = qw0 + 32 * qb;
+            bf16 *row0 = a.dq + (int64_t)b * a.dqs.b + (int64_t)head * a.dqs.h + (int64_t)r0 * a.dqs.s;
+            store_rows32(stage, dq[qb], a.scale, row0, a.dqs.s, a.Sq - r0, lane);
+            __builtin_amdgcn_wave_barrier();
+        }
     }
 }
 

@@ -66,29 +66,32 @@ __device__ __forceinline__ bf16x8 as_bf16x8(const u32x4 v) {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
-// ---- staging a 64 x 64 tile: global -> registers -> LDS, 256 threads -------------
-// Thread t owns 16-byte chunk (t % 8) of rows (t / 8) and (t / 8 + 32): eight
+// ---- staging a 64 x 64 tile: global -> registers -> LDS, NT threads --------------
+// Thread t owns 16-byte chunk (t % 8) of rows (t / 8) + k * (NT / 8): eight
 // consecutive lanes read one whole 128-byte row, so global loads are fully
 // coalesced 128-bit accesses and the LDS writes of a row are contiguous.
-struct TileRegs { u32x4 v[2]; };
+template <int NT>
+struct TileRegs { u32x4 v[512 / NT]; };
 
-__device__ __forceinline__ void tile_load(TileRegs &r, const bf16 *base, int64_t stride_s,
+template <int NT>
+__device__ __forceinline__ void tile_load(TileRegs<NT> &r, const bf16 *base, int64_t stride_s,
                                           int row0, int row_end, int tid) {
     const int c = tid & 7, rr = tid >> 3;
 #pragma unroll
-    for (int pass = 0; pass < 2; ++pass) {
-        const int row = row0 + rr + 32 * pass;
+    for (int pass = 0; pass < 512 / NT; ++pass) {
+        const int row = row0 + rr + (NT / 8) * pass;
         u32x4 z = {0u, 0u, 0u, 0u};
         if (row < row_end) z = *reinterpret_cast<const u32x4 *>(base + (int64_t)row * stride_s + c * 8);
         r.v[pass] = z;
     }
 }
 
-__device__ __forceinline__ void tile_store(bf16 *lds, const TileRegs &r, int tid) {
+template <int NT>
+__device__ __forceinline__ void tile_store(bf16 *lds, const TileRegs<NT> &r, int tid) {
     const int c = tid & 7, rr = tid >> 3;
 #pragma unroll
-    for (int pass = 0; pass < 2; ++pass)
-        *reinterpret_cast<u32x4 *>(lds + (rr + 32 * pass) * kLS + c * 8) = r.v[pass];
+    for (int pass = 0; pass < 512 / NT; ++pass)
+        *reinterpret_cast<u32x4 *>(lds + (rr + (NT / 8) * pass) * kLS + c * 8) = r.v[pass];
 }
 
 // A (or B) fragment with the contraction along head_dim: lane reads

@@ -2,27 +2,106 @@
 // row logsumexp.  Stands in for the reference's `_attn_fwd`
 // (attention_kernel.py:11-100).
 //
-// Work split.  A workgroup is 4 wavefronts.  Each wavefront owns 32 query rows
-// of ONE query head; the 4 wavefronts of a workgroup are HPB query heads of the
-// same KV head times 4/HPB consecutive 32-row slabs, so every K/V tile staged in
+// Work split.  A workgroup is 4 wavefronts.  Each wavefront owns 32*NQB query
+// rows of ONE query head; the 4 wavefronts of a workgroup are HPB query heads of
+// the same KV head times 4/HPB consecutive row slabs, so every K/V tile staged in
 // LDS is shared by the whole GQA group slice.  KV tiles are 64 keys.
 //
 // Per tile the wavefront computes S^T = K Q^T (K rows are the MFMA A operand
 // from LDS, Q^T lives in registers as the B operand), so a lane owns one query
-// row and its 32 logits sit in its own registers: the row max / row sum are
-// in-lane reductions plus one exchange with lane^32.  exp2 is used with
-// scale*log2(e) folded into one FMA.  P^T goes straight from the C registers
-// into the B operand of O^T += V^T P^T; V^T fragments come from the row-major
-// LDS tile through ds_read_b64_tr_b16.
+// row per 32-row block and its logits sit in its own registers: the row max /
+// row sum are in-lane reductions plus one exchange with lane^32.  exp2 is used
+// with scale*log2(e) folded into one FMA.  P^T goes straight from the C
+// registers into the B operand of O^T += V^T P^T; V^T fragments come from the
+// row-major LDS tile through ds_read_b64_tr_b16.  With NQB = 2 every fragment
+// read from LDS feeds two MFMAs.
 #pragma once
 #include "attn_common.h"
 
 namespace gptoss {
 
-template <int HPB>
-__global__ __launch_bounds__(256) void attn_fwd_kernel(const KArgs a) {
-    constexpr int QSUB = 4 / HPB;      // 32-row slabs per workgroup
-    constexpr int BM = 32 * QSUB;      // query rows per workgroup
+// One 64-key tile for one wavefront.  MASKED = false: every pair visible.
+// Masked variant: dbase[qb] = (lane's query position) - (first key of the tile),
+// hugely negative for a dead query row; key r of the tile is visible iff
+// 0 <= dbase - r < weff and r < key_lim.
+template <bool MASKED, int NQB>
+__device__ __forceinline__ void fwd_tile(const bf16 *ksm, const bf16 *vsm, const bf16x8 (&qf)[NQB][4],
+                                         f32x16 (&o)[NQB][2], float (&m)[NQB], float (&l)[NQB], float c, int lane,
+                                         const int (&dbase)[NQB], unsigned weff, int key_lim) {
+    const int half = lane >> 5;
+    f32x16 s[2][NQB];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+        for (int qb = 0; qb < NQB; ++qb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) s[kb][qb][i] = 0.0f;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            const bf16x8 ak = frag_nat(ksm, kb, ks, lane);
+#pragma unroll
+            for (int qb = 0; qb < NQB; ++qb) s[kb][qb] = mfma_bf16(ak, qf[qb][ks], s[kb][qb]);
+        }
+    }
+#pragma unroll
+    for (int qb = 0; qb < NQB; ++qb) {
+        if (MASKED) {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int r = 32 * kb + crow(i, half);
+                    const bool vis = ((unsigned)(dbase[qb] - r) < weff) & (r < key_lim);
+                    s[kb][qb][i] = vis ? s[kb][qb][i] : -INFINITY;
+                }
+        }
+        float mx = fmaxf(s[0][qb][0], s[1][qb][0]);
+#pragma unroll
+        for (int i = 1; i < 16; ++i) mx = fmaxf(mx, fmaxf(s[0][qb][i], s[1][qb][i]));
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float m_new = fmaxf(m[qb], mx * c);
+        if (__builtin_amdgcn_ballot_w64(m_new != m[qb]) != 0ull) {
+            const float alpha = fast_exp2(m[qb] - m_new);
+            l[qb] *= alpha;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) { o[qb][0][i] *= alpha; o[qb][1][i] *= alpha; }
+            m[qb] = m_new;
+        }
+        float rs = 0.0f;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const float pe = fast_exp2(fmaf(s[kb][qb][i], c, -m[qb]));
+                s[kb][qb][i] = pe;
+                rs += pe;
+            }
+        l[qb] += rs;
+    }
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            bf16x8 av[2];
+#pragma unroll
+            for (int dblk = 0; dblk < 2; ++dblk) av[dblk] = frag_tr(vsm, kb, u, dblk, lane);
+#pragma unroll
+            for (int qb = 0; qb < NQB; ++qb) {
+                const bf16x8 pf = cfrag(s[kb][qb], u);
+#pragma unroll
+                for (int dblk = 0; dblk < 2; ++dblk) o[qb][dblk] = mfma_bf16(av[dblk], pf, o[qb][dblk]);
+            }
+        }
+}
+
+#ifndef GPTOSS_FWD_WAVES
+#define GPTOSS_FWD_WAVES 2
+#endif
+template <int HPB, int NQB>
+__global__ __launch_bounds__(256, GPTOSS_FWD_WAVES) void attn_fwd_kernel(const KArgs a) {
+    constexpr int QSUB = 4 / HPB;      // row slabs per workgroup
+    constexpr int WM = 32 * NQB;       // query rows per wavefront
+    constexpr int BM = WM * QSUB;      // query rows per workgroup
     __shared__ __attribute__((aligned(16))) bf16 smem[2][2][kTileElems];
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
@@ -43,7 +122,7 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const KArgs a) {
     const int hsel = hc * HPB + (w % HPB);
     const bool active = hsel < a.r;
     const int head = g * a.r + (active ? hsel : 0);
-    const int qw0 = qt * BM + 32 * (w / HPB);          // first query row of this wavefront
+    const int qw0 = qt * BM + WM * (w / HPB);          // first query row of this wavefront
 
     const int kv_len = a.seqlens ? min(a.Skv, a.seqlens[b]) : a.Skv;
     const int q_len = a.seqlens ? a.seqlens[b] : 0x7fffffff;
@@ -59,120 +138,89 @@ __global__ __launch_bounds__(256) void attn_fwd_kernel(const KArgs a) {
 
     // this wavefront's own row range (absolute positions)
     const int wpos0 = a.q_offset + qw0;
-    const int wpos1 = min(a.q_offset + min(a.Sq, qw0 + 32) - 1, q_len - 1);
-    const int p = wpos0 + l32;                          // this lane's query position
-    const bool p_ok = (qw0 + l32 < a.Sq) && (p < q_len);
+    const int wpos1 = min(a.q_offset + min(a.Sq, qw0 + WM) - 1, q_len - 1);
 
     const bf16 *kbase = a.k + (int64_t)b * a.ks.b + (int64_t)g * a.ks.h;
     const bf16 *vbase = a.v + (int64_t)b * a.vs.b + (int64_t)g * a.vs.h;
 
     // Q^T fragments (B operand), resident for the whole key loop
-    bf16x8 qf[4];
-    {
-        const bf16 *qrow = a.q + (int64_t)b * a.qs.b + (int64_t)head * a.qs.h + (int64_t)(qw0 + l32) * a.qs.s;
+    bf16x8 qf[NQB][4];
+    int pq[NQB];            // lane's query position per block, hugely negative when the row is dead
+#pragma unroll
+    for (int qb = 0; qb < NQB; ++qb) {
+        const int row = qw0 + 32 * qb + l32;
+        const bf16 *qrow = a.q + (int64_t)b * a.qs.b + (int64_t)head * a.qs.h + (int64_t)row * a.qs.s;
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
             u32x4 z = {0u, 0u, 0u, 0u};
-            if (qw0 + l32 < a.Sq) z = *reinterpret_cast<const u32x4 *>(qrow + 16 * ks + 8 * half);
-            qf[ks] = as_bf16x8(z);
+            if (row < a.Sq) z = *reinterpret_cast<const u32x4 *>(qrow + 16 * ks + 8 * half);
+            qf[qb][ks] = as_bf16x8(z);
         }
+        const int p = a.q_offset + row;
+        pq[qb] = (row < a.Sq && p < q_len) ? p : -0x40000000;
     }
 
     const float c = a.scale_log2;
     const float sink2 = (a.sinks ? a.sinks[head] : 0.0f) * kLog2e;
-    float m = sink2;       // running max, log2 domain; starts at the sink logit (ref :53)
-    float l = 0.0f;        // this lane's share of the running sum (own keys only)
-    f32x16 o[2];
+    float m[NQB], l[NQB];  // running max (log2 domain, starts at the sink logit, ref :53) and
+                           // this lane's share of the running sum (own keys only)
+    f32x16 o[NQB][2];
 #pragma unroll
-    for (int i = 0; i < 16; ++i) { o[0][i] = 0.0f; o[1][i] = 0.0f; }
+    for (int qb = 0; qb < NQB; ++qb) {
+        m[qb] = sink2;
+        l[qb] = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) { o[qb][0][i] = 0.0f; o[qb][1][i] = 0.0f; }
+    }
 
-    TileRegs kr, vr;
+    TileRegs<256> kr, vr;
     if (t_lo < t_hi) {
-        tile_load(kr, kbase, a.ks.s, t_lo * kTile, a.Skv, tid);
-        tile_load(vr, vbase, a.vs.s, t_lo * kTile, a.Skv, tid);
+        tile_load<256>(kr, kbase, a.ks.s, t_lo * kTile, a.Skv, tid);
+        tile_load<256>(vr, vbase, a.vs.s, t_lo * kTile, a.Skv, tid);
     }
 
     for (int t = t_lo; t < t_hi; ++t) {
         const int buf = (t - t_lo) & 1;
         bf16 *ksm = smem[buf][0], *vsm = smem[buf][1];
-        tile_store(ksm, kr, tid);
-        tile_store(vsm, vr, tid);
+        tile_store<256>(ksm, kr, tid);
+        tile_store<256>(vsm, vr, tid);
         __syncthreads();
         if (t + 1 < t_hi) {
-            tile_load(kr, kbase, a.ks.s, (t + 1) * kTile, a.Skv, tid);
-            tile_load(vr, vbase, a.vs.s, (t + 1) * kTile, a.Skv, tid);
+            tile_load<256>(kr, kbase, a.ks.s, (t + 1) * kTile, a.Skv, tid);
+            tile_load<256>(vr, vbase, a.vs.s, (t + 1) * kTile, a.Skv, tid);
         }
         const int n0 = t * kTile;
         // tile classification for this wavefront: skip / interior / needs mask
         const bool skip = !active || n0 > wpos1 || (n0 + kTile - 1) < (wpos0 - weff + 1) || wpos1 < wpos0;
         if (skip) continue;
         const bool interior = (n0 + kTile - 1 <= wpos0) && (n0 > wpos1 - weff) && (n0 + kTile <= kv_len) &&
-                              (a.q_offset + qw0 + 31 <= wpos1);
-
-        f32x16 s[2];
+                              (a.q_offset + qw0 + WM - 1 <= wpos1);
+        if (interior) {
+            fwd_tile<false, NQB>(ksm, vsm, qf, o, m, l, c, lane, pq, 0u, 0);
+        } else {
+            int dbase[NQB];
 #pragma unroll
-        for (int blk = 0; blk < 2; ++blk) {
-#pragma unroll
-            for (int i = 0; i < 16; ++i) s[blk][i] = 0.0f;
-#pragma unroll
-            for (int ks = 0; ks < 4; ++ks) s[blk] = mfma_bf16(frag_nat(ksm, blk, ks, lane), qf[ks], s[blk]);
+            for (int qb = 0; qb < NQB; ++qb) dbase[qb] = pq[qb] - n0;   // stays hugely negative for dead rows
+            fwd_tile<true, NQB>(ksm, vsm, qf, o, m, l, c, lane, dbase, (unsigned)weff, kv_len - n0);
         }
-        if (!interior) {
-#pragma unroll
-            for (int blk = 0; blk < 2; ++blk)
-#pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const int j = n0 + 32 * blk + crow(i, half);
-                    const bool vis = p_ok && (j <= p) && (j > p - weff) && (j < kv_len);
-                    s[blk][i] = vis ? s[blk][i] : -INFINITY;
-                }
-        }
-        float mx = s[0][0];
-#pragma unroll
-        for (int i = 1; i < 16; ++i) mx = fmaxf(mx, s[0][i]);
-#pragma unroll
-        for (int i = 0; i < 16; ++i) mx = fmaxf(mx, s[1][i]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m, mx * c);
-        if (__builtin_amdgcn_ballot_w64(m_new != m) != 0ull) {
-            const float alpha = fast_exp2(m - m_new);
-            l *= alpha;
-#pragma unroll
-            for (int i = 0; i < 16; ++i) { o[0][i] *= alpha; o[1][i] *= alpha; }
-            m = m_new;
-        }
-        float rs = 0.0f;
-#pragma unroll
-        for (int blk = 0; blk < 2; ++blk)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const float pe = fast_exp2(fmaf(s[blk][i], c, -m));
-                s[blk][i] = pe;
-                rs += pe;
-            }
-        l += rs;
-#pragma unroll
-        for (int blk = 0; blk < 2; ++blk)
-#pragma unroll
-            for (int u = 0; u < 2; ++u) {
-                const bf16x8 pf = cfrag(s[blk], u);
-#pragma unroll
-                for (int dblk = 0; dblk < 2; ++dblk)
-                    o[dblk] = mfma_bf16(frag_tr(vsm, blk, u, dblk, lane), pf, o[dblk]);
-            }
     }
 
     // epilogue: z = l + exp(sink - m); O = acc / z; M = m + log z   (ref :93-98)
-    const float l_tot = l + __shfl_xor(l, 32);
-    const float z = l_tot + fast_exp2(sink2 - m);
-    const float inv = 1.0f / z;
     __syncthreads();   // every wavefront is done reading the K/V buffers
-    if (active) {
-        bf16 *stage = &smem[0][0][0] + w * 32 * kLS;
-        bf16 *orow0 = a.o + (int64_t)b * a.os.b + (int64_t)head * a.os.h + (int64_t)qw0 * a.os.s;
-        store_rows32(stage, o, inv, orow0, a.os.s, a.Sq - qw0, lane);
-        if (half == 0 && qw0 + l32 < a.Sq)
-            a.lse[((int64_t)b * a.H + head) * a.Sq + qw0 + l32] = (m + fast_log2(z)) * kLn2;
+    bf16 *stage = &smem[0][0][0] + w * 32 * kLS;
+#pragma unroll
+    for (int qb = 0; qb < NQB; ++qb) {
+        const float l_tot = l[qb] + __shfl_xor(l[qb], 32);
+        const float z = l_tot + fast_exp2(sink2 - m[qb]);
+        const float inv = 1.0f / z;
+        if (active) {
+            const int r0 = qw0 + 32 * qb;
+            bf16 *orow0 = a.o + (int64_t)b * a.os.b + (int64_t)head * a.os.h + (int64_t)r0 * a.os.s;
+            store_rows32(stage, o[qb], inv, orow0, a.os.s, a.Sq - r0, lane);
+            __builtin_amdgcn_wave_barrier();
+            if (half == 0 && r0 + l32 < a.Sq)
+                a.lse[((int64_t)b * a.H + head) * a.Sq + r0 + l32] = (m[qb] + fast_log2(z)) * kLn2;
+        }
     }
 }
 

@@ -54,6 +54,20 @@ KArgs make_args(const gptoss_attn_params *p) {
 
 int hpb_for(int r) { return r >= 4 ? 4 : (r >= 2 ? 2 : 1); }
 
+// 32-row query blocks per wavefront in the forward and dQ kernels
+#ifndef GPTOSS_FWD_QB
+#define GPTOSS_FWD_QB 2
+#endif
+#ifndef GPTOSS_DQ_QB
+#define GPTOSS_DQ_QB 1
+#endif
+#ifndef GPTOSS_DKDV_NB
+#define GPTOSS_DKDV_NB 1
+#endif
+constexpr int kDkdvNB = GPTOSS_DKDV_NB;
+constexpr int kFwdQB = GPTOSS_FWD_QB;
+constexpr int kDqQB = GPTOSS_DQ_QB;
+
 int launch_status() {
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? GPTOSS_ATTN_OK : static_cast<int>(e);
@@ -112,12 +126,12 @@ int gptoss_attn_fwd(const gptoss_attn_params *p, void *stream) {
     const KArgs a = make_args(p);
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int hpb = hpb_for(a.r);
-    const int bm = 32 * (4 / hpb);
+    const int bm = 32 * kFwdQB * (4 / hpb);
     const int n_hc = (a.r + hpb - 1) / hpb;
     const unsigned grid = (unsigned)(a.G * n_hc * a.B * ((a.Sq + bm - 1) / bm));
-    if (hpb == 4) hipLaunchKernelGGL(attn_fwd_kernel<4>, dim3(grid), dim3(256), 0, st, a);
-    else if (hpb == 2) hipLaunchKernelGGL(attn_fwd_kernel<2>, dim3(grid), dim3(256), 0, st, a);
-    else hipLaunchKernelGGL(attn_fwd_kernel<1>, dim3(grid), dim3(256), 0, st, a);
+    if (hpb == 4) hipLaunchKernelGGL((attn_fwd_kernel<4, kFwdQB>), dim3(grid), dim3(256), 0, st, a);
+    else if (hpb == 2) hipLaunchKernelGGL((attn_fwd_kernel<2, kFwdQB>), dim3(grid), dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((attn_fwd_kernel<1, kFwdQB>), dim3(grid), dim3(256), 0, st, a);
     return launch_status();
 }
 
@@ -142,8 +156,10 @@ int gptoss_attn_bwd_dkdv(const gptoss_attn_params *p, void *stream) {
     if (rc) return rc;
     const KArgs a = make_args(p);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const unsigned grid = (unsigned)(a.G * a.B * ((a.Skv + 127) / 128));
-    hipLaunchKernelGGL(attn_bwd_dkdv_kernel, dim3(grid), dim3(256), 0, st, a);
+    constexpr int kWaves = 4;                       // wavefronts per workgroup
+    const int bn = 32 * kDkdvNB * kWaves;           // keys per workgroup
+    const unsigned grid = (unsigned)(a.G * a.B * ((a.Skv + bn - 1) / bn));
+    hipLaunchKernelGGL((attn_bwd_dkdv_kernel<kWaves, kDkdvNB>), dim3(grid), dim3(64 * kWaves), 0, st, a);
     return launch_status();
 }
 
@@ -153,12 +169,12 @@ int gptoss_attn_bwd_dq(const gptoss_attn_params *p, void *stream) {
     const KArgs a = make_args(p);
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int hpb = hpb_for(a.r);
-    const int bm = 32 * (4 / hpb);
+    const int bm = 32 * kDqQB * (4 / hpb);
     const int n_hc = (a.r + hpb - 1) / hpb;
     const unsigned grid = (unsigned)(a.G * n_hc * a.B * ((a.Sq + bm - 1) / bm));
-    if (hpb == 4) hipLaunchKernelGGL(attn_bwd_dq_kernel<4>, dim3(grid), dim3(256), 0, st, a);
-    else if (hpb == 2) hipLaunchKernelGGL(attn_bwd_dq_kernel<2>, dim3(grid), dim3(256), 0, st, a);
-    else hipLaunchKernelGGL(attn_bwd_dq_kernel<1>, dim3(grid), dim3(256), 0, st, a);
+    if (hpb == 4) hipLaunchKernelGGL((attn_bwd_dq_kernel<4, kDqQB>), dim3(grid), dim3(256), 0, st, a);
+    else if (hpb == 2) hipLaunchKernelGGL((attn_bwd_dq_kernel<2, kDqQB>), dim3(grid), dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((attn_bwd_dq_kernel<1, kDqQB>), dim3(grid), dim3(256), 0, st, a);
     return launch_status();
 }
 
