@@ -65,7 +65,7 @@ def main():
         o = torch.empty((B, S, H, D), dtype=q.dtype, device=dev)
         lse = torch.empty((B, H, S), dtype=torch.float32, device=dev)
         dq, dk, dv = torch.empty_like(q), torch.empty(k.shape, dtype=k.dtype, device=dev), torch.empty(k.shape, dtype=k.dtype, device=dev)
-        delta = torch.empty((B, H, S), dtype=torch.float32, device=dev)
+        delta = torch.empty((2, B, H, S), dtype=torch.float32, device=dev)
         dsinks = torch.empty((H,), dtype=torch.float32, device=dev)
         s32 = sinks.float().contiguous()
         p = ak._base_params(q, k, v, s32, None, scale, window, 0)

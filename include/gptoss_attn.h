@@ -25,7 +25,8 @@
  *                                  (attention_kernel.py:36,152)
  *   o, d_o       (B, Sq, H, D) by default in the caller's view, but addressed
  *                through the same (b, h, s) stride triple, so any layout works
- *   lse, delta   (B, H, Sq) fp32 contiguous
+ *   lse          (B, H, Sq) fp32 contiguous
+ *   delta        fp32 scratch of 2*B*H*Sq elements: rowsum(dO*O), then lse*log2(e)
  *   sinks, dsinks (H,) fp32;  sinks == NULL means a sink logit of 0, as in the
  *                reference (attention_kernel.py:39-42)
  *   seqlens      (B,) int32 or NULL: right-padding lengths.  Keys at or beyond
@@ -88,7 +89,7 @@ typedef struct gptoss_attn_params {
     const void *d_o;
     void *dq, *dk, *dv;
     float *dsinks;          /* optional: NULL skips the sink gradient */
-    float *delta;           /* (B,H,Sq) fp32 scratch written by bwd_preprocess */
+    float *delta;           /* 2*B*H*Sq fp32 scratch written by bwd_preprocess */
 
     gptoss_attn_strides q_stride, k_stride, v_stride, o_stride;
     gptoss_attn_strides do_stride, dq_stride, dk_stride, dv_stride;
@@ -109,7 +110,8 @@ const char *gptoss_attn_status_string(int status);
 int gptoss_attn_fwd(const gptoss_attn_params *params, void *stream);
 
 /*
- * Backward step 1: delta = rowsum(dO * O).  Replaces `_attn_bwd_precompute_D`
+ * Backward step 1: delta = rowsum(dO * O) (first B*H*Sq floats of `delta`) and
+ * lse * log2(e) (the next B*H*Sq floats).  Replaces `_attn_bwd_precompute_D`
  * (attention_kernel.py:102-120, 304-313) including the dO transpose copy at
  * :290.  When dsinks != NULL it also produces
  * dsinks[h] = -sum_{b,i} exp(sinks[h] - lse) * delta   (attention_kernel.py:173-176)

@@ -125,7 +125,7 @@ def attention_backward(q, k, v, sinks, o, lse, d_o, sm_scale, window=None, q_off
     dq = torch.empty((b, h, sq, d), dtype=q.dtype, device=q.device)
     dk = torch.empty(k.shape, dtype=k.dtype, device=q.device)
     dv = torch.empty(v.shape, dtype=v.dtype, device=q.device)
-    delta = torch.empty((b, h, sq), dtype=torch.float32, device=q.device)
+    delta = torch.empty((2, b, h, sq), dtype=torch.float32, device=q.device)   # [delta; lse*log2e]
     dsinks = torch.empty((h,), dtype=torch.float32, device=q.device) if need_dsinks else None
     with torch.cuda.device(q.device):
         p = _base_params(q, k, v, sinks32, sl, sm_scale, window, q_offset)

@@ -8,6 +8,8 @@
 //                           tile) that can see them                      (:199-212)
 //   attn_bwd_dq_kernel      Q-outer, same shape as the forward kernel    (:206-217)
 #pragma once
+#include <type_traits>
+
 #include "attn_common.h"
 
 // Scheduling fence between software-pipeline phases (keeps early-issued LDS reads early).
@@ -20,8 +22,11 @@
 namespace gptoss {
 
 // ---------------------------------------------------------------------------------
-// delta[b,h,s] = sum_d dO[b,h,s,d] * O[b,h,s,d].  HBM-bound stream: eight lanes
-// read one 128-byte row of each tensor, reduce with three xor-shuffles.
+// -delta[b,h,s] = -sum_d dO[b,h,s,d] * O[b,h,s,d] (negated so that the dK/dV kernel can
+// load it straight into the dP accumulators).  HBM-bound stream: eight lanes
+// read one 128-byte row of each tensor, reduce with three xor-shuffles.  The same
+// pass stores lse*log2(e) in the second half of the scratch buffer, which is what
+// the dK/dV and dQ kernels feed to exp2.
 __global__ __launch_bounds__(256) void attn_bwd_delta_kernel(const KArgs a) {
     const int64_t rid = (int64_t)blockIdx.x * 32 + (threadIdx.x >> 3);   // (b*H + h)*Sq + s
     const int64_t total = (int64_t)a.B * a.H * a.Sq;
@@ -39,7 +44,10 @@ __global__ __launch_bounds__(256) void attn_bwd_delta_kernel(const KArgs a) {
     acc += __shfl_xor(acc, 1);
     acc += __shfl_xor(acc, 2);
     acc += __shfl_xor(acc, 4);
-    if (c == 0) a.delta[rid] = acc;
+    if (c == 0) {
+        a.delta[rid] = -acc;                          // stored negated: it seeds the dP accumulators
+        a.delta[total + rid] = a.lse[rid] * kLog2e;   // second half of the scratch: lse in log2 units
+    }
 }
 
 // ---------------------------------------------------------------------------------
@@ -54,7 +62,7 @@ __global__ __launch_bounds__(256) void attn_bwd_dsinks_kernel(const KArgs a) {
         const float *lse = a.lse + ((int64_t)b * a.H + h) * a.Sq;
         const float *dl = a.delta + ((int64_t)b * a.H + h) * a.Sq;
         for (int s = threadIdx.x; s < a.Sq; s += 256)
-            acc -= fast_exp2(sink2 - lse[s] * kLog2e) * dl[s];
+            acc += fast_exp2(sink2 - lse[s] * kLog2e) * dl[s];   // dl holds -delta
     }
     red[threadIdx.x] = acc;
     __syncthreads();
@@ -82,90 +90,81 @@ __global__ __launch_bounds__(256) void attn_bwd_dsinks_kernel(const KArgs a) {
 // is visible iff 0 <= dbase + r < weff, tested with one unsigned compare; rows at
 // or beyond `row_lim` (relative to the tile) do not exist.
 template <bool MASKED, int NB>
-__device__ __forceinline__ void dkdv_tile(const bf16 *qsm, const bf16 *gsm, const float *lse_s, const float *del_s,
+__device__ __forceinline__ void dkdv_tile(uint32_t qsm, uint32_t gsm, uint32_t stat_lane, const TileLaneOffsets &lo,
                                           const bf16x8 (&kf)[NB][4], const bf16x8 (&vf)[NB][4],
-                                          f32x16 (&dk)[NB][2], f32x16 (&dv)[NB][2], float c, int lane,
+                                          f32x16 (&dk)[NB][2], f32x16 (&dv)[NB][2], float c, int half,
                                           const int (&dbase)[NB], unsigned weff, int row_lim) {
-    const int half = lane >> 5;
-    // LDS reads are issued one phase ahead of the MFMAs that consume them, so the
-    // matrix pipe never waits on an LDS round trip:
-    //   [A frags of block qb] -> S/dP MFMAs -> [transposed frags + row stats] ->
-    //   exp / dS on the VALU (A frags of block qb+1 in flight) -> dV/dK MFMAs.
-    bf16x8 aq[4], ag[4];
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) { aq[ks] = frag_nat(qsm, 0, ks, lane); ag[ks] = frag_nat(gsm, 0, ks, lane); }
+    // qsm / gsm: LDS byte addresses of the staged Q and dO tiles; stat_lane: address of this
+    // lane's first lse2 value (rows 4*half..), -delta sits kTile floats further on.
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) {
         f32x16 s[NB], dp[NB];
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-            for (int i = 0; i < 16; ++i) { s[nb][i] = 0.0f; dp[nb][i] = 0.0f; }
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb) {
-                s[nb] = mfma_bf16(aq[ks], kf[nb][ks], s[nb]);
-                dp[nb] = mfma_bf16(ag[ks], vf[nb][ks], dp[nb]);
-            }
-        GPTOSS_SCHED_FENCE();
-        bf16x8 agt[2][2], aqt[2][2];
-#pragma unroll
-        for (int u = 0; u < 2; ++u)
-#pragma unroll
-            for (int dblk = 0; dblk < 2; ++dblk) {
-                agt[u][dblk] = frag_tr(gsm, qb, u, dblk, lane);
-                aqt[u][dblk] = frag_tr(qsm, qb, u, dblk, lane);
-            }
-        f32x4 lv[4], dl[4];
+        // the dP accumulators start at -delta of their rows, so the MFMAs deliver dP - delta
 #pragma unroll
         for (int a4 = 0; a4 < 4; ++a4) {
-            lv[a4] = *reinterpret_cast<const f32x4 *>(lse_s + 32 * qb + 8 * a4 + 4 * half);
-            dl[a4] = *reinterpret_cast<const f32x4 *>(del_s + 32 * qb + 8 * a4 + 4 * half);
-        }
-        if (qb == 0) {
+            const f32x4 nd = lds_load128f(stat_lane, (kTile + 32 * qb + 8 * a4) * 4);
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks) { aq[ks] = frag_nat(qsm, 1, ks, lane); ag[ks] = frag_nat(gsm, 1, ks, lane); }
-        }
-        GPTOSS_SCHED_FENCE();
+            for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-        for (int a4 = 0; a4 < 4; ++a4)
+                for (int e = 0; e < 4; ++e) { s[nb][4 * a4 + e] = 0.0f; dp[nb][4 * a4 + e] = nd[e]; }
+        }
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            const bf16x8 aq = ofrag_nat(qsm, lo, qb, ks);
+            const bf16x8 ag = ofrag_nat(gsm, lo, qb, ks);
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                s[nb] = mfma_bf16(aq, kf[nb][ks], s[nb]);
+                dp[nb] = mfma_bf16(ag, vf[nb][ks], dp[nb]);
+            }
+        }
+#pragma unroll
+        for (int a4 = 0; a4 < 4; ++a4) {
+            const f32x4 lv = lds_load128f(stat_lane, (32 * qb + 8 * a4) * 4);
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int i = 4 * a4 + e;
-                    float pe = fast_exp2(fmaf(s[nb][i], c, -lv[a4][e]));
+                    float pe = fast_exp2(fmaf(s[nb][i], c, -lv[e]));
                     if (MASKED) {
                         const int r = 32 * qb + 8 * a4 + 4 * half + e;
                         const bool vis = ((unsigned)(dbase[nb] + r) < weff) & (r < row_lim);
                         pe = vis ? pe : 0.0f;
                     }
                     s[nb][i] = pe;
-                    dp[nb][i] = pe * (dp[nb][i] - dl[a4][e]);
+                    dp[nb][i] = pe * dp[nb][i];
                 }
-        GPTOSS_SCHED_FENCE();
+        }
 #pragma unroll
-        for (int u = 0; u < 2; ++u)
+        for (int u = 0; u < 2; ++u) {
+            bf16x8 agt[2], aqt[2];
+#pragma unroll
+            for (int dblk = 0; dblk < 2; ++dblk) {
+                agt[dblk] = ofrag_tr(gsm, lo, qb, u, dblk);
+                aqt[dblk] = ofrag_tr(qsm, lo, qb, u, dblk);
+            }
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) {
                 const bf16x8 pf = cfrag(s[nb], u), dsf = cfrag(dp[nb], u);
 #pragma unroll
                 for (int dblk = 0; dblk < 2; ++dblk) {
-                    dv[nb][dblk] = mfma_bf16(agt[u][dblk], pf, dv[nb][dblk]);
-                    dk[nb][dblk] = mfma_bf16(aqt[u][dblk], dsf, dk[nb][dblk]);
+                    dv[nb][dblk] = mfma_bf16(agt[dblk], pf, dv[nb][dblk]);
+                    dk[nb][dblk] = mfma_bf16(aqt[dblk], dsf, dk[nb][dblk]);
                 }
             }
+        }
     }
 }
 
 template <int NW, int NB>             // NB = 32-key blocks per wavefront
 __global__ __launch_bounds__(NW * 64, (NB == 1 ? 2 : 1)) void attn_bwd_dkdv_kernel(const KArgs a) {
-    constexpr int NT = NW * 64;
+    static_assert(NW == 4, "the asynchronous tile copy is written for 4 wavefronts");
+    constexpr int NS = 3;              // LDS stages: tiles are requested two iterations ahead
     constexpr int WK = 32 * NB;        // keys per wavefront
     constexpr int BN = WK * NW;        // keys per workgroup
-    __shared__ __attribute__((aligned(16))) bf16 smem[2][2][kTileElems];
-    __shared__ __attribute__((aligned(16))) float sstat[2][2][kTile];
+    __shared__ __attribute__((aligned(16))) char smem[NS][2][kStageTileBytes];
+    __shared__ __attribute__((aligned(16))) float sstat[NS][2][kTile];
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int l32 = lane & 31, half = lane >> 5;
@@ -221,43 +220,51 @@ __global__ __launch_bounds__(NW * 64, (NB == 1 ? 2 : 1)) void attn_bwd_dkdv_kern
     int dead[NB];
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) dead[nb] = 0;
-    TileRegs<NT> qr, gr;
-    float st = 0.0f;     // lse*log2e (threads 0..63) or delta (threads 64..127) of the staged tile
+    const float *lse2 = a.delta + (int64_t)a.B * a.H * a.Sq;   // written by the delta kernel
+    const TileLaneOffsets lo = make_tile_offsets(lane);
+    const uint32_t smem_base = lds_addr(&smem[0][0][0]), stat_base = lds_addr(&sstat[0][0][0]);
 
-    auto prefetch = [&](int it) {
-        const int hq = g * a.r + it / nq;
-        const int i0 = (qt_lo + it % nq) * kTile;
-        tile_load<NT>(qr, a.q + (int64_t)b * a.qs.b + (int64_t)hq * a.qs.h, a.qs.s, i0, a.Sq, tid);
-        tile_load<NT>(gr, a.d_o + (int64_t)b * a.dos.b + (int64_t)hq * a.dos.h, a.dos.s, i0, a.Sq, tid);
-        if (tid < 128) {
-            const int i = i0 + (tid & 63);
-            const int64_t off = ((int64_t)b * a.H + hq) * a.Sq + i;
-            st = 0.0f;
-            if (i < a.Sq) st = (tid < 64) ? a.lse[off] * kLog2e : a.delta[off];
+    // Iteration `it` -> (query tile, query head).  Query tiles run from the LAST one
+    // down and heads are the inner index, so every workgroup of this KV head that is
+    // resident at the same time walks the same Q / dO tiles in the same order and finds
+    // them in its XCD's L2.
+    auto issue = [&](int it) {
+        const int stage = it % NS;
+        const int hq = g * a.r + it % a.r;
+        const int i0 = (qt_hi - 1 - it / a.r) * kTile;
+        tile_async(smem[stage][0], a.q + (int64_t)b * a.qs.b + (int64_t)hq * a.qs.h, a.qs.s, i0, a.Sq, lane, w);
+        tile_async(smem[stage][1], a.d_o + (int64_t)b * a.dos.b + (int64_t)hq * a.dos.h, a.dos.s, i0, a.Sq, lane, w);
+        // row statistics: wavefront w copies 32 floats of lse2 (w < 2) or delta (w >= 2)
+        if (lane < 32) {
+            const int i = min(i0 + 32 * (w & 1) + lane, a.Sq - 1);
+            const float *src = ((w >> 1) ? a.delta : lse2) + ((int64_t)b * a.H + hq) * a.Sq + i;
+            __builtin_amdgcn_global_load_lds((glb_void_t *)src, (lds_void_t *)(&sstat[stage][w >> 1][32 * (w & 1)]), 4, 0, 0);
         }
     };
+    constexpr int kLoadsPerIt = 5;     // vector-memory instructions one wavefront issues per iteration
 
-    if (n_it > 0) prefetch(0);
-    for (int it = 0; it < n_it; ++it) {
-        const int buf = it & 1;
-        bf16 *qsm = smem[buf][0], *gsm = smem[buf][1];
-        tile_store<NT>(qsm, qr, tid);
-        tile_store<NT>(gsm, gr, tid);
-        if (tid < 128) sstat[buf][tid >> 6][tid & 63] = st;
+    // One iteration on a compile-time LDS stage, so that every fragment address is
+    // (lane offset register) + (immediate).
+    auto iterate = [&](int it, auto stage_tag) {
+        constexpr int STAGE = decltype(stage_tag)::value;
+        // the copies for this iteration were issued two iterations ago; those of the next
+        // one may stay in flight
+        if (it + 1 < n_it) wait_vmcnt<kLoadsPerIt>(); else wait_vmcnt<0>();
         __syncthreads();
-        if (it + 1 < n_it) prefetch(it + 1);
+        if (it + 2 < n_it) issue(it + 2);
 
-        const int i0 = (qt_lo + it % nq) * kTile;
+        const uint32_t qsm = smem_base + STAGE * (2 * kStageTileBytes), gsm = qsm + kStageTileBytes;
+        const uint32_t stat_lane = stat_base + STAGE * (2 * kTile * 4) + half * 16;
+        const int i0 = (qt_hi - 1 - it / a.r) * kTile;
         const int pos0 = a.q_offset + i0;                                    // first query position of the tile
         const int pos1 = min(a.q_offset + min(a.Sq, i0 + kTile) - 1, q_len - 1);   // last live one
         const int wj1 = min(wj0 + WK, kv_len) - 1;                           // wavefront's last live key
         const bool skip = wj1 < wj0 || pos1 < wj0 || pos0 > wj1 + weff - 1 || pos1 < pos0;
-        if (skip) continue;
+        if (skip) return;
         const bool interior = (wj0 + WK - 1 <= pos0) && (wj0 > pos1 - weff) && (wj0 + WK <= kv_len) &&
                               (a.q_offset + i0 + kTile - 1 <= pos1);
-        const float *lse_s = sstat[buf][0], *del_s = sstat[buf][1];
         if (interior) {
-            dkdv_tile<false, NB>(qsm, gsm, lse_s, del_s, kf, vf, dk, dv, c, lane, dead, 0u, 0);
+            dkdv_tile<false, NB>(qsm, gsm, stat_lane, lo, kf, vf, dk, dv, c, half, dead, 0u, 0);
         } else {
             int dbase[NB];
 #pragma unroll
@@ -266,20 +273,28 @@ __global__ __launch_bounds__(NW * 64, (NB == 1 ? 2 : 1)) void attn_bwd_dkdv_kern
                 dbase[nb] = (j < kv_len) ? pos0 - j : -0x40000000;
             }
             const int row_lim = (int)min((int64_t)kTile, min((int64_t)a.Sq, (int64_t)q_len - a.q_offset) - i0);
-            dkdv_tile<true, NB>(qsm, gsm, lse_s, del_s, kf, vf, dk, dv, c, lane, dbase, (unsigned)weff, row_lim);
+            dkdv_tile<true, NB>(qsm, gsm, stat_lane, lo, kf, vf, dk, dv, c, half, dbase, (unsigned)weff, row_lim);
         }
+    };
+
+    if (n_it > 0) issue(0);
+    if (n_it > 1) issue(1);
+    for (int it = 0; it < n_it; it += NS) {
+        iterate(it, std::integral_constant<int, 0>{});
+        if (it + 1 < n_it) iterate(it + 1, std::integral_constant<int, 1>{});
+        if (it + 2 < n_it) iterate(it + 2, std::integral_constant<int, 2>{});
     }
 
     __syncthreads();
-    bf16 *stage = &smem[0][0][0] + w * 32 * kLS;
+    bf16 *stage_out = reinterpret_cast<bf16 *>(&smem[0][0][0]) + w * 32 * kLS;
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
         const int r0 = wj0 + 32 * nb;
         const int nvalid = a.Skv - r0;
-        store_rows32(stage, dk[nb], a.scale, a.dk + (int64_t)b * a.dks.b + (int64_t)g * a.dks.h + (int64_t)r0 * a.dks.s,
+        store_rows32(stage_out, dk[nb], a.scale, a.dk + (int64_t)b * a.dks.b + (int64_t)g * a.dks.h + (int64_t)r0 * a.dks.s,
                      a.dks.s, nvalid, lane);
         __builtin_amdgcn_wave_barrier();
-        store_rows32(stage, dv[nb], 1.0f, a.dv + (int64_t)b * a.dvs.b + (int64_t)g * a.dvs.h + (int64_t)r0 * a.dvs.s,
+        store_rows32(stage_out, dv[nb], 1.0f, a.dv + (int64_t)b * a.dvs.b + (int64_t)g * a.dvs.h + (int64_t)r0 * a.dvs.s,
                      a.dvs.s, nvalid, lane);
         __builtin_amdgcn_wave_barrier();
     }
@@ -291,7 +306,7 @@ __global__ __launch_bounds__(NW * 64, (NB == 1 ? 2 : 1)) void attn_bwd_dkdv_kern
 //   S^T = K Q^T, dP^T = V dO^T, P = exp2(S*c - lse*log2e), dS = P (dP - delta),
 //   dQ^T += K^T dS^T   (A = transposed read of the K tile, B = C registers).
 template <bool MASKED, int NQB>
-__device__ __forceinline__ void dq_tile(const bf16 *ksm, const bf16 *vsm, const bf16x8 (&qf)[NQB][4],
+__device__ __forceinline__ void dq_tile(uint32_t ksm, uint32_t vsm, const TileLaneOffsets &lo, const bf16x8 (&qf)[NQB][4],
                                         const bf16x8 (&gf)[NQB][4], f32x16 (&dq)[NQB][2], const float (&lse2)[NQB],
                                         const float (&dlt)[NQB], float c, int lane, const int (&dbase)[NQB],
                                         unsigned weff, int key_lim) {
@@ -305,8 +320,8 @@ __device__ __forceinline__ void dq_tile(const bf16 *ksm, const bf16 *vsm, const 
             for (int i = 0; i < 16; ++i) { s[qb][i] = 0.0f; dp[qb][i] = 0.0f; }
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
-            const bf16x8 ak = frag_nat(ksm, kb, ks, lane);
-            const bf16x8 av = frag_nat(vsm, kb, ks, lane);
+            const bf16x8 ak = ofrag_nat(ksm, lo, kb, ks);
+            const bf16x8 av = ofrag_nat(vsm, lo, kb, ks);
 #pragma unroll
             for (int qb = 0; qb < NQB; ++qb) {
                 s[qb] = mfma_bf16(ak, qf[qb][ks], s[qb]);
@@ -323,13 +338,13 @@ __device__ __forceinline__ void dq_tile(const bf16 *ksm, const bf16 *vsm, const 
                     const bool vis = ((unsigned)(dbase[qb] - r) < weff) & (r < key_lim);
                     pe = vis ? pe : 0.0f;
                 }
-                dp[qb][i] = pe * (dp[qb][i] - dlt[qb]);
+                dp[qb][i] = pe * (dp[qb][i] + dlt[qb]);        // dlt holds -delta
             }
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             bf16x8 akt[2];
 #pragma unroll
-            for (int dblk = 0; dblk < 2; ++dblk) akt[dblk] = frag_tr(ksm, kb, u, dblk, lane);
+            for (int dblk = 0; dblk < 2; ++dblk) akt[dblk] = ofrag_tr(ksm, lo, kb, u, dblk);
 #pragma unroll
             for (int qb = 0; qb < NQB; ++qb) {
                 const bf16x8 dsf = cfrag(dp[qb], u);
@@ -341,14 +356,15 @@ __device__ __forceinline__ void dq_tile(const bf16 *ksm, const bf16 *vsm, const 
 }
 
 #ifndef GPTOSS_DQ_WAVES
-#define GPTOSS_DQ_WAVES 3
+#define GPTOSS_DQ_WAVES 2
 #endif
 template <int HPB, int NQB>
 __global__ __launch_bounds__(256, GPTOSS_DQ_WAVES) void attn_bwd_dq_kernel(const KArgs a) {
     constexpr int QSUB = 4 / HPB;
     constexpr int WM = 32 * NQB;
     constexpr int BM = WM * QSUB;
-    __shared__ __attribute__((aligned(16))) bf16 smem[2][2][kTileElems];
+    constexpr int NS = 3;
+    __shared__ __attribute__((aligned(16))) char smem[NS][2][kStageTileBytes];
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int l32 = lane & 31, half = lane >> 5;
@@ -373,8 +389,8 @@ __global__ __launch_bounds__(256, GPTOSS_DQ_WAVES) void attn_bwd_dq_kernel(const
     const int bpos0 = a.q_offset + qt * BM;
     const int bpos1 = min(a.q_offset + min(a.Sq, (qt + 1) * BM) - 1, q_len - 1);
     const int hi = bpos1 >= bpos0 ? min(kv_len, bpos1 + 1) : 0;
-    const int lo = max(0, bpos0 - weff + 1);
-    const int t_lo = lo / kTile;
+    const int key_lo = max(0, bpos0 - weff + 1);
+    const int t_lo = key_lo / kTile;
     const int t_hi = hi > 0 ? (hi + kTile - 1) / kTile : 0;
 
     const int wpos0 = a.q_offset + qw0;
@@ -420,38 +436,47 @@ __global__ __launch_bounds__(256, GPTOSS_DQ_WAVES) void attn_bwd_dq_kernel(const
 #pragma unroll
         for (int i = 0; i < 16; ++i) { dq[qb][0][i] = 0.0f; dq[qb][1][i] = 0.0f; }
 
-    TileRegs<256> kr, vr;
-    if (t_lo < t_hi) {
-        tile_load<256>(kr, kbase, a.ks.s, t_lo * kTile, a.Skv, tid);
-        tile_load<256>(vr, vbase, a.vs.s, t_lo * kTile, a.Skv, tid);
-    }
-    for (int t = t_lo; t < t_hi; ++t) {
-        const int buf = (t - t_lo) & 1;
-        bf16 *ksm = smem[buf][0], *vsm = smem[buf][1];
-        tile_store<256>(ksm, kr, tid);
-        tile_store<256>(vsm, vr, tid);
+    const TileLaneOffsets lo = make_tile_offsets(lane);
+    const uint32_t smem_base = lds_addr(&smem[0][0][0]);
+    const int n_it = max(0, t_hi - t_lo);
+    auto issue = [&](int it) {
+        const int stage = it % NS;
+        tile_async(smem[stage][0], kbase, a.ks.s, (t_lo + it) * kTile, a.Skv, lane, w);
+        tile_async(smem[stage][1], vbase, a.vs.s, (t_lo + it) * kTile, a.Skv, lane, w);
+    };
+    constexpr int kLoadsPerIt = 4;
+
+    auto iterate = [&](int it, auto stage_tag) {
+        constexpr int STAGE = decltype(stage_tag)::value;
+        if (it + 1 < n_it) wait_vmcnt<kLoadsPerIt>(); else wait_vmcnt<0>();
         __syncthreads();
-        if (t + 1 < t_hi) {
-            tile_load<256>(kr, kbase, a.ks.s, (t + 1) * kTile, a.Skv, tid);
-            tile_load<256>(vr, vbase, a.vs.s, (t + 1) * kTile, a.Skv, tid);
-        }
-        const int n0 = t * kTile;
+        if (it + 2 < n_it) issue(it + 2);
+        const uint32_t ksm = smem_base + STAGE * (2 * kStageTileBytes), vsm = ksm + kStageTileBytes;
+        const int n0 = (t_lo + it) * kTile;
         const bool skip = !active || n0 > wpos1 || (n0 + kTile - 1) < (wpos0 - weff + 1) || wpos1 < wpos0;
-        if (skip) continue;
+        if (skip) return;
         const bool interior = (n0 + kTile - 1 <= wpos0) && (n0 > wpos1 - weff) && (n0 + kTile <= kv_len) &&
                               (a.q_offset + qw0 + WM - 1 <= wpos1);
         if (interior) {
-            dq_tile<false, NQB>(ksm, vsm, qf, gf, dq, lse2, dlt, c, lane, pq, 0u, 0);
+            dq_tile<false, NQB>(ksm, vsm, lo, qf, gf, dq, lse2, dlt, c, lane, pq, 0u, 0);
         } else {
             int dbase[NQB];
 #pragma unroll
             for (int qb = 0; qb < NQB; ++qb) dbase[qb] = pq[qb] - n0;
-            dq_tile<true, NQB>(ksm, vsm, qf, gf, dq, lse2, dlt, c, lane, dbase, (unsigned)weff, kv_len - n0);
+            dq_tile<true, NQB>(ksm, vsm, lo, qf, gf, dq, lse2, dlt, c, lane, dbase, (unsigned)weff, kv_len - n0);
         }
+    };
+
+    if (n_it > 0) issue(0);
+    if (n_it > 1) issue(1);
+    for (int it = 0; it < n_it; it += NS) {
+        iterate(it, std::integral_constant<int, 0>{});
+        if (it + 1 < n_it) iterate(it + 1, std::integral_constant<int, 1>{});
+        if (it + 2 < n_it) iterate(it + 2, std::integral_constant<int, 2>{});
     }
     __syncthreads();
     if (active) {
-        bf16 *stage = &smem[0][0][0] + w * 32 * kLS;
+        bf16 *stage = reinterpret_cast<bf16 *>(&smem[0][0][0]) + w * 32 * kLS;
 #pragma unroll
         for (int qb = 0; qb < NQB; ++qb) {
             const int r0 = qw0 + 32 * qb;

@@ -131,6 +131,126 @@ __device__ __forceinline__ bf16x8 cfrag(const f32x16 &c, int u) {
     return f;
 }
 
+// ---- asynchronous tile staging: global -> LDS without passing through registers ----
+// global_load_lds_dwordx4 writes lane L's 16 bytes at (wave-uniform LDS base) + 16*L,
+// so one instruction fills 8 unpadded 128-byte rows.  To keep the later fragment reads
+// free of bank conflicts the 16-byte chunks of a row are XOR-swizzled: physical chunk p
+// of tile row r holds logical chunk p ^ swz(r).  swz() is chosen so that
+//   * 16 consecutive rows reading the same logical chunk (natural 128-bit fragment
+//     reads) fall in 16 distinct 16-byte bank groups, and
+//   * 4 consecutive rows x 2 adjacent chunks (transposing 64-bit reads) do as well.
+constexpr int kRowBytes = kD * 2;                 // 128
+constexpr int kStageTileBytes = kTile * kRowBytes; // 8192
+
+__device__ __forceinline__ int swz(int r) { return (((r >> 1) & 1) << 2) | (((r >> 3) & 1) << 1) | ((r >> 2) & 1); }
+
+typedef __attribute__((address_space(3))) void lds_void_t;
+typedef __attribute__((address_space(1))) const void glb_void_t;
+
+// Issues the 4-wavefront asynchronous copy of tile rows [row0, row0+64) (rows at or
+// beyond row_end re-read the last valid row: their products are masked, they only
+// have to be finite).  Each wavefront issues two instructions.
+__device__ __forceinline__ void tile_async(char *lds_tile, const bf16 *base, int64_t stride_s, int row0,
+                                           int row_end, int lane, int w) {
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        const int r = 16 * w + 8 * k + (lane >> 3);
+        const int c = (lane & 7) ^ swz(r);
+        const int row = min(row0 + r, row_end - 1);
+        const bf16 *src = base + (int64_t)row * stride_s + c * 8;
+        __builtin_amdgcn_global_load_lds((glb_void_t *)src, (lds_void_t *)(lds_tile + (16 * w + 8 * k) * kRowBytes), 16, 0, 0);
+    }
+}
+
+// Waits until at most `n` of this wavefront's vector-memory operations are outstanding.
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+    static_assert(N >= 0 && N < 64, "vmcnt range");
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
+}
+
+// Fragment readers for a swizzled tile (same fragment contents as frag_nat / frag_tr).
+__device__ __forceinline__ bf16x8 sfrag_nat(const char *tile, int blk, int ks, int lane) {
+    const int row = 32 * blk + (lane & 31);
+    const int c = (2 * ks + (lane >> 5)) ^ swz(row);
+    return as_bf16x8(*reinterpret_cast<const u32x4 *>(tile + row * kRowBytes + c * 16));
+}
+
+__device__ __forceinline__ bf16x8 sfrag_tr(const char *tile, int blk, int u, int dblk, int lane) {
+    const int i = lane & 15, g16 = lane >> 4, half = g16 >> 1;
+    const int row = 32 * blk + 16 * u + 4 * half + (i >> 2);
+    const int chunk = 4 * dblk + 2 * (g16 & 1) + ((i & 3) >> 1);
+    const int sub = (i & 1) * 8;
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    const char *p0 = tile + row * kRowBytes + ((chunk ^ swz(row)) * 16) + sub;
+    const char *p1 = tile + (row + 8) * kRowBytes + ((chunk ^ swz(row + 8)) * 16) + sub;
+    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(p0));
+    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(p1));
+    union { struct { s16x4 a, b; } s; bf16x8 v; } x;
+    x.s.a = lo; x.s.b = hi;
+    return x.v;
+}
+
+// ---- register-cheap addressing of swizzled tiles --------------------------------
+// All lane-dependent parts of the fragment addresses are computed once per kernel
+// (TileLaneOffsets); inside the loops an address is (stage base + lane offset) with
+// the block / tile selection folded into the instruction's immediate offset.
+typedef __attribute__((address_space(3))) char lds_char_t;
+
+__device__ __forceinline__ uint32_t lds_addr(const void *p) {
+    return (uint32_t)(uintptr_t)(lds_char_t *)p;
+}
+__device__ __forceinline__ u32x4 lds_load128(uint32_t addr, int imm) {
+    return *reinterpret_cast<const __attribute__((address_space(3))) u32x4 *>((uintptr_t)(addr + imm));
+}
+__device__ __forceinline__ f32x4 lds_load128f(uint32_t addr, int imm) {
+    return *reinterpret_cast<const __attribute__((address_space(3))) f32x4 *>((uintptr_t)(addr + imm));
+}
+__device__ __forceinline__ s16x4 lds_load_tr64(uint32_t addr, int imm) {
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(uintptr_t)(addr + imm));
+}
+
+struct TileLaneOffsets {
+    uint32_t nat[4];      // [ks]: natural fragment, row l32 of block 0
+    uint32_t tr[2][2];    // [dblk][t]: transposed fragment, u = 0 of block 0, rows (+8*t)
+};
+
+__device__ __forceinline__ TileLaneOffsets make_tile_offsets(int lane) {
+    TileLaneOffsets o;
+    {
+        const int row = lane & 31;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) o.nat[ks] = row * kRowBytes + (((2 * ks + (lane >> 5)) ^ swz(row)) * 16);
+    }
+    {
+        const int i = lane & 15, g16 = lane >> 4, half = g16 >> 1;
+        const int sub = (i & 1) * 8;
+#pragma unroll
+        for (int dblk = 0; dblk < 2; ++dblk)
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {
+                const int row = 4 * half + (i >> 2) + 8 * t;
+                const int chunk = 4 * dblk + 2 * (g16 & 1) + ((i & 3) >> 1);
+                o.tr[dblk][t] = row * kRowBytes + ((chunk ^ swz(row)) * 16) + sub;
+            }
+    }
+    return o;
+}
+
+// natural fragment of 32-row block `blk`; `tile` = LDS byte address of the tile
+__device__ __forceinline__ bf16x8 ofrag_nat(uint32_t tile, const TileLaneOffsets &o, int blk, int ks) {
+    return as_bf16x8(lds_load128(tile + o.nat[ks], blk * 32 * kRowBytes));
+}
+// transposed fragment: rows 32*blk + 16*u + {4*half + 0..3, 8 + 4*half + 0..3}, columns 32*dblk + l32
+__device__ __forceinline__ bf16x8 ofrag_tr(uint32_t tile, const TileLaneOffsets &o, int blk, int u, int dblk) {
+    const int imm = (32 * blk + 16 * u) * kRowBytes;
+    union { struct { s16x4 a, b; } s; bf16x8 v; } x;
+    x.s.a = lds_load_tr64(tile + o.tr[dblk][0], imm);
+    x.s.b = lds_load_tr64(tile + o.tr[dblk][1], imm);
+    return x.v;
+}
+
 // Writes a wave's 32 x 64 result held as two transposed accumulators
 // (lane = row l32, register i of acc[dblk] = column 32*dblk + crow(i, half)) to
 // global memory through a wave-private LDS stage so that the global stores are

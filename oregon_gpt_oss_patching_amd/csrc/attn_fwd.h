@@ -16,6 +16,8 @@
 // row-major LDS tile through ds_read_b64_tr_b16.  With NQB = 2 every fragment
 // read from LDS feeds two MFMAs.
 #pragma once
+#include <type_traits>
+
 #include "attn_common.h"
 
 namespace gptoss {
@@ -25,7 +27,7 @@ namespace gptoss {
 // hugely negative for a dead query row; key r of the tile is visible iff
 // 0 <= dbase - r < weff and r < key_lim.
 template <bool MASKED, int NQB>
-__device__ __forceinline__ void fwd_tile(const bf16 *ksm, const bf16 *vsm, const bf16x8 (&qf)[NQB][4],
+__device__ __forceinline__ void fwd_tile(uint32_t ksm, uint32_t vsm, const TileLaneOffsets &lo, const bf16x8 (&qf)[NQB][4],
                                          f32x16 (&o)[NQB][2], float (&m)[NQB], float (&l)[NQB], float c, int lane,
                                          const int (&dbase)[NQB], unsigned weff, int key_lim) {
     const int half = lane >> 5;
@@ -38,7 +40,7 @@ __device__ __forceinline__ void fwd_tile(const bf16 *ksm, const bf16 *vsm, const
             for (int i = 0; i < 16; ++i) s[kb][qb][i] = 0.0f;
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
-            const bf16x8 ak = frag_nat(ksm, kb, ks, lane);
+            const bf16x8 ak = ofrag_nat(ksm, lo, kb, ks);
 #pragma unroll
             for (int qb = 0; qb < NQB; ++qb) s[kb][qb] = mfma_bf16(ak, qf[qb][ks], s[kb][qb]);
         }
@@ -84,7 +86,7 @@ __device__ __forceinline__ void fwd_tile(const bf16 *ksm, const bf16 *vsm, const
         for (int u = 0; u < 2; ++u) {
             bf16x8 av[2];
 #pragma unroll
-            for (int dblk = 0; dblk < 2; ++dblk) av[dblk] = frag_tr(vsm, kb, u, dblk, lane);
+            for (int dblk = 0; dblk < 2; ++dblk) av[dblk] = ofrag_tr(vsm, lo, kb, u, dblk);
 #pragma unroll
             for (int qb = 0; qb < NQB; ++qb) {
                 const bf16x8 pf = cfrag(s[kb][qb], u);
@@ -102,7 +104,8 @@ __global__ __launch_bounds__(256, GPTOSS_FWD_WAVES) void attn_fwd_kernel(const K
     constexpr int QSUB = 4 / HPB;      // row slabs per workgroup
     constexpr int WM = 32 * NQB;       // query rows per wavefront
     constexpr int BM = WM * QSUB;      // query rows per workgroup
-    __shared__ __attribute__((aligned(16))) bf16 smem[2][2][kTileElems];
+    constexpr int NS = 3;              // LDS stages: K/V tiles are requested two iterations ahead
+    __shared__ __attribute__((aligned(16))) char smem[NS][2][kStageTileBytes];
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int l32 = lane & 31, half = lane >> 5;
@@ -132,8 +135,8 @@ __global__ __launch_bounds__(256, GPTOSS_FWD_WAVES) void attn_fwd_kernel(const K
     const int bpos0 = a.q_offset + qt * BM;
     const int bpos1 = min(a.q_offset + min(a.Sq, (qt + 1) * BM) - 1, q_len - 1);
     const int hi = bpos1 >= bpos0 ? min(kv_len, bpos1 + 1) : 0;   // no key at all for a fully padded tile
-    const int lo = max(0, bpos0 - weff + 1);
-    const int t_lo = lo / kTile;
+    const int key_lo = max(0, bpos0 - weff + 1);
+    const int t_lo = key_lo / kTile;
     const int t_hi = hi > 0 ? (hi + kTile - 1) / kTile : 0;
 
     // this wavefront's own row range (absolute positions)
@@ -173,41 +176,49 @@ __global__ __launch_bounds__(256, GPTOSS_FWD_WAVES) void attn_fwd_kernel(const K
         for (int i = 0; i < 16; ++i) { o[qb][0][i] = 0.0f; o[qb][1][i] = 0.0f; }
     }
 
-    TileRegs<256> kr, vr;
-    if (t_lo < t_hi) {
-        tile_load<256>(kr, kbase, a.ks.s, t_lo * kTile, a.Skv, tid);
-        tile_load<256>(vr, vbase, a.vs.s, t_lo * kTile, a.Skv, tid);
-    }
+    const TileLaneOffsets lo = make_tile_offsets(lane);
+    const uint32_t smem_base = lds_addr(&smem[0][0][0]);
+    const int n_it = max(0, t_hi - t_lo);
+    auto issue = [&](int it) {
+        const int stage = it % NS;
+        tile_async(smem[stage][0], kbase, a.ks.s, (t_lo + it) * kTile, a.Skv, lane, w);
+        tile_async(smem[stage][1], vbase, a.vs.s, (t_lo + it) * kTile, a.Skv, lane, w);
+    };
+    constexpr int kLoadsPerIt = 4;     // vector-memory instructions one wavefront issues per iteration
 
-    for (int t = t_lo; t < t_hi; ++t) {
-        const int buf = (t - t_lo) & 1;
-        bf16 *ksm = smem[buf][0], *vsm = smem[buf][1];
-        tile_store<256>(ksm, kr, tid);
-        tile_store<256>(vsm, vr, tid);
+    auto iterate = [&](int it, auto stage_tag) {
+        constexpr int STAGE = decltype(stage_tag)::value;
+        if (it + 1 < n_it) wait_vmcnt<kLoadsPerIt>(); else wait_vmcnt<0>();
         __syncthreads();
-        if (t + 1 < t_hi) {
-            tile_load<256>(kr, kbase, a.ks.s, (t + 1) * kTile, a.Skv, tid);
-            tile_load<256>(vr, vbase, a.vs.s, (t + 1) * kTile, a.Skv, tid);
-        }
-        const int n0 = t * kTile;
+        if (it + 2 < n_it) issue(it + 2);
+        const uint32_t ksm = smem_base + STAGE * (2 * kStageTileBytes), vsm = ksm + kStageTileBytes;
+        const int n0 = (t_lo + it) * kTile;
         // tile classification for this wavefront: skip / interior / needs mask
         const bool skip = !active || n0 > wpos1 || (n0 + kTile - 1) < (wpos0 - weff + 1) || wpos1 < wpos0;
-        if (skip) continue;
+        if (skip) return;
         const bool interior = (n0 + kTile - 1 <= wpos0) && (n0 > wpos1 - weff) && (n0 + kTile <= kv_len) &&
                               (a.q_offset + qw0 + WM - 1 <= wpos1);
         if (interior) {
-            fwd_tile<false, NQB>(ksm, vsm, qf, o, m, l, c, lane, pq, 0u, 0);
+            fwd_tile<false, NQB>(ksm, vsm, lo, qf, o, m, l, c, lane, pq, 0u, 0);
         } else {
             int dbase[NQB];
 #pragma unroll
             for (int qb = 0; qb < NQB; ++qb) dbase[qb] = pq[qb] - n0;   // stays hugely negative for dead rows
-            fwd_tile<true, NQB>(ksm, vsm, qf, o, m, l, c, lane, dbase, (unsigned)weff, kv_len - n0);
+            fwd_tile<true, NQB>(ksm, vsm, lo, qf, o, m, l, c, lane, dbase, (unsigned)weff, kv_len - n0);
         }
+    };
+
+    if (n_it > 0) issue(0);
+    if (n_it > 1) issue(1);
+    for (int it = 0; it < n_it; it += NS) {
+        iterate(it, std::integral_constant<int, 0>{});
+        if (it + 1 < n_it) iterate(it + 1, std::integral_constant<int, 1>{});
+        if (it + 2 < n_it) iterate(it + 2, std::integral_constant<int, 2>{});
     }
 
     // epilogue: z = l + exp(sink - m); O = acc / z; M = m + log z   (ref :93-98)
     __syncthreads();   // every wavefront is done reading the K/V buffers
-    bf16 *stage = &smem[0][0][0] + w * 32 * kLS;
+    bf16 *stage = reinterpret_cast<bf16 *>(&smem[0][0][0]) + w * 32 * kLS;
 #pragma unroll
     for (int qb = 0; qb < NQB; ++qb) {
         const float l_tot = l[qb] + __shfl_xor(l[qb], 32);

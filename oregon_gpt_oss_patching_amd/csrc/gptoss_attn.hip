@@ -59,7 +59,7 @@ int hpb_for(int r) { return r >= 4 ? 4 : (r >= 2 ? 2 : 1); }
 #define GPTOSS_FWD_QB 2
 #endif
 #ifndef GPTOSS_DQ_QB
-#define GPTOSS_DQ_QB 1
+#define GPTOSS_DQ_QB 2
 #endif
 #ifndef GPTOSS_DKDV_NB
 #define GPTOSS_DKDV_NB 1
