@@ -26,6 +26,7 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2516.6   # MI355X dense bf16 MFMA peak
 PEAK_HBM_GBS = 8000.0
+DKDV_HBM_BYTES_S16K = int((713948.3 * 2.0 + 32768.0) * 1024)   # measured, see profiles/
 
 
 def pairs(s, w):
@@ -40,6 +41,10 @@ def main():
     ap.add_argument("--seq", type=int, default=16384)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-seq", type=int, default=16384, help="sequence length of the CPU-baseline sample")
+    ap.add_argument("--layers", choices=("both", "full", "window"), default="both",
+                    help="which layer types to run (profiling runs use one, so per-kernel averages are unmixed)")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run a plain 1 GiB device copy, the known-size kernel that HBM byte counters are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the attention op has no cross-GPU "
@@ -65,7 +70,7 @@ def main():
         o = torch.empty((B, S, H, D), dtype=q.dtype, device=dev)
         lse = torch.empty((B, H, S), dtype=torch.float32, device=dev)
         dq, dk, dv = torch.empty_like(q), torch.empty(k.shape, dtype=k.dtype, device=dev), torch.empty(k.shape, dtype=k.dtype, device=dev)
-        delta = torch.empty((2, B, H, S), dtype=torch.float32, device=dev)
+        delta = torch.empty((2, B, H, S), dtype=torch.float32, device=dev)   # [-delta; lse*log2e]
         dsinks = torch.empty((H,), dtype=torch.float32, device=dev)
         s32 = sinks.float().contiguous()
         p = ak._base_params(q, k, v, s32, None, scale, window, 0)
@@ -114,6 +119,21 @@ def main():
     p_full, keep_full = make_params(0)
     p_win, keep_win = make_params(128)
 
+    if args.copy_calibration:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
+    if args.layers != "both":
+        # profiling mode: run the chosen layer type only and report its step time
+        p = p_full if args.layers == "full" else p_win
+        ms = time_steps(p, args.steps, args.warmup)
+        print(json.dumps({"layers": args.layers, "ms_per_step": round(ms, 4), "steps": args.steps}))
+        return
+
     ms_full = time_steps(p_full, args.steps, args.warmup)
     ms_win = time_steps(p_win, args.steps, args.warmup)
 
@@ -157,7 +177,10 @@ def main():
         "kernel_ms": kern,
         "roofline": {"bound": "mfma", "kernel": "attn_bwd_dkdv_kernel (full causal)",
                      "achieved": round(dkdv_tflops, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(dkdv_tflops / PEAK_BF16_TFLOPS, 4), "traffic": None},
+                     "frac": round(dkdv_tflops / PEAK_BF16_TFLOPS, 4),
+                     # HBM bytes per launch of this kernel at S=16384 from rocprofv3 --pmc FETCH_SIZE (x2.0) and
+                     # WRITE_SIZE (x1.0), factors from a plain 1 GiB copy kernel; only valid for the default shape
+                     "traffic": DKDV_HBM_BYTES_S16K if S == 16384 else None},
     }
 
     if not args.no_cpu_baseline:
