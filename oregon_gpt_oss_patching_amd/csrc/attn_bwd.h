@@ -28,45 +28,58 @@ namespace gptoss {
 // pass stores lse*log2(e) in the second half of the scratch buffer, which is what
 // the dK/dV and dQ kernels feed to exp2.
 __global__ __launch_bounds__(256) void attn_bwd_delta_kernel(const KArgs a) {
-    const int64_t rid = (int64_t)blockIdx.x * 32 + (threadIdx.x >> 3);   // (b*H + h)*Sq + s
-    const int64_t total = (int64_t)a.B * a.H * a.Sq;
-    if (rid >= total) return;
+    constexpr int kRowsPerThread = 4;                      // independent 128-bit loads in flight per tensor
+    const int64_t total = (int64_t)a.B * a.H * a.Sq;       // rows, indexed (b*H + h)*Sq + s
     const int c = threadIdx.x & 7;
-    const int s = (int)(rid % a.Sq);
-    const int bh = (int)(rid / a.Sq);
-    const int h = bh % a.H, b = bh / a.H;
-    const u32x4 ov = *reinterpret_cast<const u32x4 *>(a.o + (int64_t)b * a.os.b + (int64_t)h * a.os.h + (int64_t)s * a.os.s + c * 8);
-    const u32x4 gv = *reinterpret_cast<const u32x4 *>(a.d_o + (int64_t)b * a.dos.b + (int64_t)h * a.dos.h + (int64_t)s * a.dos.s + c * 8);
-    const bf16x8 of = as_bf16x8(ov), gf = as_bf16x8(gv);
-    float acc = 0.0f;
+    const int64_t rid0 = (int64_t)blockIdx.x * (32 * kRowsPerThread) + (threadIdx.x >> 3);
+    u32x4 ov[kRowsPerThread], gv[kRowsPerThread];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) acc = fmaf((float)of[j], (float)gf[j], acc);
-    acc += __shfl_xor(acc, 1);
-    acc += __shfl_xor(acc, 2);
-    acc += __shfl_xor(acc, 4);
-    if (c == 0) {
-        a.delta[rid] = -acc;                          // stored negated: it seeds the dP accumulators
-        a.delta[total + rid] = a.lse[rid] * kLog2e;   // second half of the scratch: lse in log2 units
+    for (int k = 0; k < kRowsPerThread; ++k) {
+        const int64_t rid = rid0 + 32 * k;
+        ov[k] = u32x4{0u, 0u, 0u, 0u};
+        gv[k] = u32x4{0u, 0u, 0u, 0u};
+        if (rid < total) {
+            const int s = (int)(rid % a.Sq);
+            const int bh = (int)(rid / a.Sq);
+            const int h = bh % a.H, b = bh / a.H;
+            ov[k] = *reinterpret_cast<const u32x4 *>(a.o + (int64_t)b * a.os.b + (int64_t)h * a.os.h + (int64_t)s * a.os.s + c * 8);
+            gv[k] = *reinterpret_cast<const u32x4 *>(a.d_o + (int64_t)b * a.dos.b + (int64_t)h * a.dos.h + (int64_t)s * a.dos.s + c * 8);
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < kRowsPerThread; ++k) {
+        const int64_t rid = rid0 + 32 * k;
+        const bf16x8 of = as_bf16x8(ov[k]), gf = as_bf16x8(gv[k]);
+        float acc = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc = fmaf((float)of[j], (float)gf[j], acc);
+        acc += __shfl_xor(acc, 1);
+        acc += __shfl_xor(acc, 2);
+        acc += __shfl_xor(acc, 4);
+        if (c == 0 && rid < total) {
+            a.delta[rid] = -acc;                          // stored negated: it seeds the dP accumulators
+            a.delta[total + rid] = a.lse[rid] * kLog2e;   // second half of the scratch: lse in log2 units
+        }
     }
 }
 
 // ---------------------------------------------------------------------------------
 // One workgroup per query head; fixed summation order, so the result is
 // bit-reproducible (the reference accumulates it with relaxed atomics).
-__global__ __launch_bounds__(256) void attn_bwd_dsinks_kernel(const KArgs a) {
-    __shared__ float red[256];
+__global__ __launch_bounds__(1024) void attn_bwd_dsinks_kernel(const KArgs a) {
+    __shared__ float red[1024];
     const int h = blockIdx.x;
     const float sink2 = (a.sinks ? a.sinks[h] : 0.0f) * kLog2e;
+    const int64_t total = (int64_t)a.B * a.H * a.Sq;
     float acc = 0.0f;
     for (int b = 0; b < a.B; ++b) {
-        const float *lse = a.lse + ((int64_t)b * a.H + h) * a.Sq;
-        const float *dl = a.delta + ((int64_t)b * a.H + h) * a.Sq;
-        for (int s = threadIdx.x; s < a.Sq; s += 256)
-            acc += fast_exp2(sink2 - lse[s] * kLog2e) * dl[s];   // dl holds -delta
+        const float *ndl = a.delta + ((int64_t)b * a.H + h) * a.Sq;        // -delta
+        const float *lse2 = ndl + total;                                    // lse * log2(e)
+        for (int s = threadIdx.x; s < a.Sq; s += 1024) acc += fast_exp2(sink2 - lse2[s]) * ndl[s];
     }
     red[threadIdx.x] = acc;
     __syncthreads();
-    for (int off = 128; off > 0; off >>= 1) {
+    for (int off = 512; off > 0; off >>= 1) {
         if ((int)threadIdx.x < off) red[threadIdx.x] += red[threadIdx.x + off];
         __syncthreads();
     }
@@ -93,11 +106,15 @@ template <bool MASKED, int NB>
 __device__ __forceinline__ void dkdv_tile(uint32_t qsm, uint32_t gsm, uint32_t stat_lane, const TileLaneOffsets &lo,
                                           const bf16x8 (&kf)[NB][4], const bf16x8 (&vf)[NB][4],
                                           f32x16 (&dk)[NB][2], f32x16 (&dv)[NB][2], float c, int half,
-                                          const int (&dbase)[NB], unsigned weff, int row_lim) {
+                                          const int (&dbase)[NB], unsigned weff, int row_lim, int krel) {
     // qsm / gsm: LDS byte addresses of the staged Q and dO tiles; stat_lane: address of this
     // lane's first lse2 value (rows 4*half..), -delta sits kTile floats further on.
+    // krel (masked variant only): (first key of the wavefront) - (first query position of the
+    // tile); a 32-row block whose rows all precede the keys, or all lost them from their
+    // window, is skipped.
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) {
+        if (MASKED && ((32 * qb + 31 < krel) || (32 * qb > krel + 32 * NB - 1 + (int)weff - 1) || (32 * qb >= row_lim))) continue;
         f32x16 s[NB], dp[NB];
         // the dP accumulators start at -delta of their rows, so the MFMAs deliver dP - delta
 #pragma unroll
@@ -264,7 +281,7 @@ __global__ __launch_bounds__(NW * 64, (NB == 1 ? 2 : 1)) void attn_bwd_dkdv_kern
         const bool interior = (wj0 + WK - 1 <= pos0) && (wj0 > pos1 - weff) && (wj0 + WK <= kv_len) &&
                               (a.q_offset + i0 + kTile - 1 <= pos1);
         if (interior) {
-            dkdv_tile<false, NB>(qsm, gsm, stat_lane, lo, kf, vf, dk, dv, c, half, dead, 0u, 0);
+            dkdv_tile<false, NB>(qsm, gsm, stat_lane, lo, kf, vf, dk, dv, c, half, dead, 0u, 0, 0);
         } else {
             int dbase[NB];
 #pragma unroll
@@ -273,7 +290,7 @@ __global__ __launch_bounds__(NW * 64, (NB == 1 ? 2 : 1)) void attn_bwd_dkdv_kern
                 dbase[nb] = (j < kv_len) ? pos0 - j : -0x40000000;
             }
             const int row_lim = (int)min((int64_t)kTile, min((int64_t)a.Sq, (int64_t)q_len - a.q_offset) - i0);
-            dkdv_tile<true, NB>(qsm, gsm, stat_lane, lo, kf, vf, dk, dv, c, half, dbase, (unsigned)weff, row_lim);
+            dkdv_tile<true, NB>(qsm, gsm, stat_lane, lo, kf, vf, dk, dv, c, half, dbase, (unsigned)weff, row_lim, wj0 - pos0);
         }
     };
 
@@ -309,10 +326,13 @@ template <bool MASKED, int NQB>
 __device__ __forceinline__ void dq_tile(uint32_t ksm, uint32_t vsm, const TileLaneOffsets &lo, const bf16x8 (&qf)[NQB][4],
                                         const bf16x8 (&gf)[NQB][4], f32x16 (&dq)[NQB][2], const float (&lse2)[NQB],
                                         const float (&dlt)[NQB], float c, int lane, const int (&dbase)[NQB],
-                                        unsigned weff, int key_lim) {
+                                        unsigned weff, int key_lim, int wrel) {
+    // wrel (masked variant only): (first query position of the wavefront) - (first key of the
+    // tile); a 32-key half of the tile that no row of the wavefront can see is skipped.
     const int half = lane >> 5;
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
+        if (MASKED && ((32 * kb > wrel + 32 * NQB - 1) || (32 * kb + 31 < wrel - (int)weff + 1) || (32 * kb >= key_lim))) continue;
         f32x16 s[NQB], dp[NQB];
 #pragma unroll
         for (int qb = 0; qb < NQB; ++qb)
@@ -355,11 +375,8 @@ __device__ __forceinline__ void dq_tile(uint32_t ksm, uint32_t vsm, const TileLa
     }
 }
 
-#ifndef GPTOSS_DQ_WAVES
-#define GPTOSS_DQ_WAVES 2
-#endif
 template <int HPB, int NQB>
-__global__ __launch_bounds__(256, GPTOSS_DQ_WAVES) void attn_bwd_dq_kernel(const KArgs a) {
+__global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_bwd_dq_kernel(const KArgs a) {
     constexpr int QSUB = 4 / HPB;
     constexpr int WM = 32 * NQB;
     constexpr int BM = WM * QSUB;
@@ -422,8 +439,8 @@ __global__ __launch_bounds__(256, GPTOSS_DQ_WAVES) void attn_bwd_dq_kernel(const
         dlt[qb] = 0.0f;
         if (row_ok) {
             const int64_t off = ((int64_t)b * a.H + head) * a.Sq + row;
-            lse2[qb] = a.lse[off] * kLog2e;
-            dlt[qb] = a.delta[off];
+            lse2[qb] = a.delta[(int64_t)a.B * a.H * a.Sq + off];   // lse * log2(e), written by the delta kernel
+            dlt[qb] = a.delta[off];                                  // -delta
         }
         const int p = a.q_offset + row;
         pq[qb] = (row_ok && p < q_len) ? p : -0x40000000;
@@ -458,12 +475,12 @@ __global__ __launch_bounds__(256, GPTOSS_DQ_WAVES) void attn_bwd_dq_kernel(const
         const bool interior = (n0 + kTile - 1 <= wpos0) && (n0 > wpos1 - weff) && (n0 + kTile <= kv_len) &&
                               (a.q_offset + qw0 + WM - 1 <= wpos1);
         if (interior) {
-            dq_tile<false, NQB>(ksm, vsm, lo, qf, gf, dq, lse2, dlt, c, lane, pq, 0u, 0);
+            dq_tile<false, NQB>(ksm, vsm, lo, qf, gf, dq, lse2, dlt, c, lane, pq, 0u, 0, 0);
         } else {
             int dbase[NQB];
 #pragma unroll
             for (int qb = 0; qb < NQB; ++qb) dbase[qb] = pq[qb] - n0;
-            dq_tile<true, NQB>(ksm, vsm, lo, qf, gf, dq, lse2, dlt, c, lane, dbase, (unsigned)weff, kv_len - n0);
+            dq_tile<true, NQB>(ksm, vsm, lo, qf, gf, dq, lse2, dlt, c, lane, dbase, (unsigned)weff, kv_len - n0, wpos0 - n0);
         }
     };
 

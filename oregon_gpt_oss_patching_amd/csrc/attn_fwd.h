@@ -29,20 +29,29 @@ namespace gptoss {
 template <bool MASKED, int NQB>
 __device__ __forceinline__ void fwd_tile(uint32_t ksm, uint32_t vsm, const TileLaneOffsets &lo, const bf16x8 (&qf)[NQB][4],
                                          f32x16 (&o)[NQB][2], float (&m)[NQB], float (&l)[NQB], float c, int lane,
-                                         const int (&dbase)[NQB], unsigned weff, int key_lim) {
+                                         const int (&dbase)[NQB], unsigned weff, int key_lim, int wrel) {
+    // wrel (masked variant only): (first query position of the wavefront) - (first key of the
+    // tile).  A 32-key half of the tile whose keys all lie in the future of every row of the
+    // wavefront, or all fell out of every row's window, is skipped outright (no MFMA, no exp).
     const int half = lane >> 5;
+    bool dead[2];
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb)
+        dead[kb] = MASKED && ((32 * kb > wrel + 32 * NQB - 1) || (32 * kb + 31 < wrel - (int)weff + 1) || (32 * kb >= key_lim));
     f32x16 s[2][NQB];
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
         for (int qb = 0; qb < NQB; ++qb)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) s[kb][qb][i] = 0.0f;
+            for (int i = 0; i < 16; ++i) s[kb][qb][i] = dead[kb] ? -INFINITY : 0.0f;
+        if (dead[kb]) continue;
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
             const bf16x8 ak = ofrag_nat(ksm, lo, kb, ks);
 #pragma unroll
-            for (int qb = 0; qb < NQB; ++qb) s[kb][qb] = mfma_bf16(ak, qf[qb][ks], s[kb][qb]);
+            for (int qb = 0; qb < NQB; ++qb)
+                s[kb][qb] = mfma_bf16(ak, qf[qb][ks], s[kb][qb]);
         }
     }
 #pragma unroll
@@ -50,11 +59,13 @@ __device__ __forceinline__ void fwd_tile(uint32_t ksm, uint32_t vsm, const TileL
         if (MASKED) {
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
+                if (!dead[kb]) {
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    const int r = 32 * kb + crow(i, half);
-                    const bool vis = ((unsigned)(dbase[qb] - r) < weff) & (r < key_lim);
-                    s[kb][qb][i] = vis ? s[kb][qb][i] : -INFINITY;
+                    for (int i = 0; i < 16; ++i) {
+                        const int r = 32 * kb + crow(i, half);
+                        const bool vis = ((unsigned)(dbase[qb] - r) < weff) & (r < key_lim);
+                        s[kb][qb][i] = vis ? s[kb][qb][i] : -INFINITY;
+                    }
                 }
         }
         float mx = fmaxf(s[0][qb][0], s[1][qb][0]);
@@ -72,16 +83,19 @@ __device__ __forceinline__ void fwd_tile(uint32_t ksm, uint32_t vsm, const TileL
         float rs = 0.0f;
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
+            if (!dead[kb]) {
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const float pe = fast_exp2(fmaf(s[kb][qb][i], c, -m[qb]));
-                s[kb][qb][i] = pe;
-                rs += pe;
+                for (int i = 0; i < 16; ++i) {
+                    const float pe = fast_exp2(fmaf(s[kb][qb][i], c, -m[qb]));
+                    s[kb][qb][i] = pe;
+                    rs += pe;
+                }
             }
         l[qb] += rs;
     }
 #pragma unroll
-    for (int kb = 0; kb < 2; ++kb)
+    for (int kb = 0; kb < 2; ++kb) {
+        if (dead[kb]) continue;
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             bf16x8 av[2];
@@ -94,13 +108,11 @@ __device__ __forceinline__ void fwd_tile(uint32_t ksm, uint32_t vsm, const TileL
                 for (int dblk = 0; dblk < 2; ++dblk) o[qb][dblk] = mfma_bf16(av[dblk], pf, o[qb][dblk]);
             }
         }
+    }
 }
 
-#ifndef GPTOSS_FWD_WAVES
-#define GPTOSS_FWD_WAVES 2
-#endif
 template <int HPB, int NQB>
-__global__ __launch_bounds__(256, GPTOSS_FWD_WAVES) void attn_fwd_kernel(const KArgs a) {
+__global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_fwd_kernel(const KArgs a) {
     constexpr int QSUB = 4 / HPB;      // row slabs per workgroup
     constexpr int WM = 32 * NQB;       // query rows per wavefront
     constexpr int BM = WM * QSUB;      // query rows per workgroup
@@ -199,12 +211,12 @@ __global__ __launch_bounds__(256, GPTOSS_FWD_WAVES) void attn_fwd_kernel(const K
         const bool interior = (n0 + kTile - 1 <= wpos0) && (n0 > wpos1 - weff) && (n0 + kTile <= kv_len) &&
                               (a.q_offset + qw0 + WM - 1 <= wpos1);
         if (interior) {
-            fwd_tile<false, NQB>(ksm, vsm, lo, qf, o, m, l, c, lane, pq, 0u, 0);
+            fwd_tile<false, NQB>(ksm, vsm, lo, qf, o, m, l, c, lane, pq, 0u, 0, 0);
         } else {
             int dbase[NQB];
 #pragma unroll
             for (int qb = 0; qb < NQB; ++qb) dbase[qb] = pq[qb] - n0;   // stays hugely negative for dead rows
-            fwd_tile<true, NQB>(ksm, vsm, lo, qf, o, m, l, c, lane, dbase, (unsigned)weff, kv_len - n0);
+            fwd_tile<true, NQB>(ksm, vsm, lo, qf, o, m, l, c, lane, dbase, (unsigned)weff, kv_len - n0, wpos0 - n0);
         }
     };
 

@@ -54,19 +54,14 @@ KArgs make_args(const gptoss_attn_params *p) {
 
 int hpb_for(int r) { return r >= 4 ? 4 : (r >= 2 ? 2 : 1); }
 
-// 32-row query blocks per wavefront in the forward and dQ kernels
-#ifndef GPTOSS_FWD_QB
-#define GPTOSS_FWD_QB 2
-#endif
-#ifndef GPTOSS_DQ_QB
-#define GPTOSS_DQ_QB 2
-#endif
-#ifndef GPTOSS_DKDV_NB
-#define GPTOSS_DKDV_NB 1
-#endif
-constexpr int kDkdvNB = GPTOSS_DKDV_NB;
-constexpr int kFwdQB = GPTOSS_FWD_QB;
-constexpr int kDqQB = GPTOSS_DQ_QB;
+// 32-row query blocks per wavefront in the forward and dQ kernels.  Two blocks (64 rows)
+// halve the LDS fragment traffic per MFMA and win on long key loops (full-causal layers);
+// one block (32 rows, three wavefronts per SIMD) wastes less of the narrow band of a
+// sliding-window layer and hides its short loops' latency better.
+int query_blocks_for(int window) { return (window > 0 && window <= 1024) ? 1 : 2; }
+
+// 32-key blocks per wavefront in the dK/dV kernel
+constexpr int kDkdvNB = 1;
 
 int launch_status() {
     const hipError_t e = hipGetLastError();
@@ -125,13 +120,17 @@ int gptoss_attn_fwd(const gptoss_attn_params *p, void *stream) {
     if (rc) return rc;
     const KArgs a = make_args(p);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const int hpb = hpb_for(a.r);
-    const int bm = 32 * kFwdQB * (4 / hpb);
+    const int hpb = hpb_for(a.r), qb = query_blocks_for(a.window);
+    const int bm = 32 * qb * (4 / hpb);
     const int n_hc = (a.r + hpb - 1) / hpb;
-    const unsigned grid = (unsigned)(a.G * n_hc * a.B * ((a.Sq + bm - 1) / bm));
-    if (hpb == 4) hipLaunchKernelGGL((attn_fwd_kernel<4, kFwdQB>), dim3(grid), dim3(256), 0, st, a);
-    else if (hpb == 2) hipLaunchKernelGGL((attn_fwd_kernel<2, kFwdQB>), dim3(grid), dim3(256), 0, st, a);
-    else hipLaunchKernelGGL((attn_fwd_kernel<1, kFwdQB>), dim3(grid), dim3(256), 0, st, a);
+    const dim3 grid((unsigned)(a.G * n_hc * a.B * ((a.Sq + bm - 1) / bm))), block(256);
+#define GPTOSS_LAUNCH_FWD(HPB, QB) hipLaunchKernelGGL((attn_fwd_kernel<HPB, QB>), grid, block, 0, st, a)
+    if (qb == 2) {
+        if (hpb == 4) GPTOSS_LAUNCH_FWD(4, 2); else if (hpb == 2) GPTOSS_LAUNCH_FWD(2, 2); else GPTOSS_LAUNCH_FWD(1, 2);
+    } else {
+        if (hpb == 4) GPTOSS_LAUNCH_FWD(4, 1); else if (hpb == 2) GPTOSS_LAUNCH_FWD(2, 1); else GPTOSS_LAUNCH_FWD(1, 1);
+    }
+#undef GPTOSS_LAUNCH_FWD
     return launch_status();
 }
 
@@ -141,11 +140,11 @@ int gptoss_attn_bwd_preprocess(const gptoss_attn_params *p, void *stream) {
     const KArgs a = make_args(p);
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int64_t rows = (int64_t)a.B * a.H * a.Sq;
-    hipLaunchKernelGGL(attn_bwd_delta_kernel, dim3((unsigned)((rows + 31) / 32)), dim3(256), 0, st, a);
+    hipLaunchKernelGGL(attn_bwd_delta_kernel, dim3((unsigned)((rows + 127) / 128)), dim3(256), 0, st, a);
     int s = launch_status();
     if (s) return s;
     if (a.dsinks) {
-        hipLaunchKernelGGL(attn_bwd_dsinks_kernel, dim3((unsigned)a.H), dim3(256), 0, st, a);
+        hipLaunchKernelGGL(attn_bwd_dsinks_kernel, dim3((unsigned)a.H), dim3(1024), 0, st, a);
         s = launch_status();
     }
     return s;
@@ -168,13 +167,17 @@ int gptoss_attn_bwd_dq(const gptoss_attn_params *p, void *stream) {
     if (rc) return rc;
     const KArgs a = make_args(p);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const int hpb = hpb_for(a.r);
-    const int bm = 32 * kDqQB * (4 / hpb);
+    const int hpb = hpb_for(a.r), qb = query_blocks_for(a.window);
+    const int bm = 32 * qb * (4 / hpb);
     const int n_hc = (a.r + hpb - 1) / hpb;
-    const unsigned grid = (unsigned)(a.G * n_hc * a.B * ((a.Sq + bm - 1) / bm));
-    if (hpb == 4) hipLaunchKernelGGL((attn_bwd_dq_kernel<4, kDqQB>), dim3(grid), dim3(256), 0, st, a);
-    else if (hpb == 2) hipLaunchKernelGGL((attn_bwd_dq_kernel<2, kDqQB>), dim3(grid), dim3(256), 0, st, a);
-    else hipLaunchKernelGGL((attn_bwd_dq_kernel<1, kDqQB>), dim3(grid), dim3(256), 0, st, a);
+    const dim3 grid((unsigned)(a.G * n_hc * a.B * ((a.Sq + bm - 1) / bm))), block(256);
+#define GPTOSS_LAUNCH_DQ(HPB, QB) hipLaunchKernelGGL((attn_bwd_dq_kernel<HPB, QB>), grid, block, 0, st, a)
+    if (qb == 2) {
+        if (hpb == 4) GPTOSS_LAUNCH_DQ(4, 2); else if (hpb == 2) GPTOSS_LAUNCH_DQ(2, 2); else GPTOSS_LAUNCH_DQ(1, 2);
+    } else {
+        if (hpb == 4) GPTOSS_LAUNCH_DQ(4, 1); else if (hpb == 2) GPTOSS_LAUNCH_DQ(2, 1); else GPTOSS_LAUNCH_DQ(1, 1);
+    }
+#undef GPTOSS_LAUNCH_DQ
     return launch_status();
 }
 
