@@ -190,9 +190,13 @@ def hip_flash_attention(
     Like the reference it ignores `attention_mask` and `dropout`: causality and the
     sliding window come from `module.sliding_window`, the sink logits from
     `module.sinks`.  A caller with right-padded batches may pass `seqlens=` in
-    kwargs."""
-    out = attention(query, key, value, module.sinks, scaling, module.sliding_window, None,
-                    kwargs.get("seqlens"))
+    kwargs, or hand a 1-D integer tensor of valid lengths over as `attention_mask`."""
+    seqlens = kwargs.get("seqlens")
+    if (seqlens is None and torch.is_tensor(attention_mask) and attention_mask.dim() == 1
+            and not attention_mask.dtype.is_floating_point):
+        # valid lengths handed over in place of the dense mask (see sft_bench.mask_free_attention_mask)
+        seqlens = attention_mask
+    out = attention(query, key, value, module.sinks, scaling, module.sliding_window, None, seqlens)
     return out, None
 
 

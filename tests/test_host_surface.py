@@ -49,3 +49,28 @@ def test_stride_helper_layouts():
     v = t.transpose(1, 2)                     # HF's value_states view: (B, H, S, D) strides of (B,S,H,D)
     assert ak._strides_bhs(v, "bhsd") == (5 * 3 * 64, 64, 3 * 64)
     assert ak._row_contiguous(v.to(torch.bfloat16)) is not None
+
+
+def test_lora_wrapper_freezes_base_and_targets_attention_projections():
+    from oregon_gpt_oss_patching_amd import sft_bench
+    model = sft_bench.build_model(layers=2, hidden=64, heads=4, kv_heads=2, head_dim=16, experts=2, top_k=2,
+                                  vocab=128, window=8, dtype=torch.float32, device="cpu")
+    params = sft_bench.add_lora(model, r=4, alpha=8.0)
+    trainable = [n for n, p in model.named_parameters() if p.requires_grad]
+    assert len(params) == len(trainable) == 2 * 4 * 2            # A and B for q,k,v,o in 2 layers
+    assert all(".self_attn." in n and "lora_" in n for n in trainable)
+    assert model.config.layer_types == ["sliding_attention", "full_attention"]
+    # zero-initialised B: the adapter is a no-op at the start
+    attn = model.model.layers[0].self_attn
+    x = torch.randn(3, 64)
+    assert torch.equal(attn.q_proj(x), attn.q_proj.base(x))
+
+
+def test_mask_free_attention_mask_carries_lengths():
+    from oregon_gpt_oss_patching_amd import sft_bench
+    m = sft_bench.mask_free_attention_mask(None)
+    assert m == {"full_attention": None, "sliding_attention": None}
+    pad = torch.tensor([[1, 1, 1, 0], [1, 1, 1, 1]])
+    m = sft_bench.mask_free_attention_mask(pad)
+    assert m["full_attention"].tolist() == [3, 4] and m["full_attention"].dtype == torch.int32
+    assert m["sliding_attention"] is m["full_attention"]
