@@ -102,6 +102,7 @@ __global__ __launch_bounds__(1024) void attn_bwd_dsinks_kernel(const KArgs a) {
 // lane's key), or a huge negative number for a dead key, so that pair (row r, key)
 // is visible iff 0 <= dbase + r < weff, tested with one unsigned compare; rows at
 // or beyond `row_lim` (relative to the tile) do not exist.
+#ifndef GPTOSS_DKDV_PIPE
 template <bool MASKED, int NB>
 __device__ __forceinline__ void dkdv_tile(uint32_t qsm, uint32_t gsm, uint32_t stat_lane, const TileLaneOffsets &lo,
                                           const bf16x8 (&kf)[NB][4], const bf16x8 (&vf)[NB][4],
@@ -174,6 +175,86 @@ __device__ __forceinline__ void dkdv_tile(uint32_t qsm, uint32_t gsm, uint32_t s
     }
 }
 
+#else
+template <bool MASKED, int NB>
+__device__ __forceinline__ void dkdv_tile(uint32_t qsm, uint32_t gsm, uint32_t stat_lane, const TileLaneOffsets &lo,
+                                          const bf16x8 (&kf)[NB][4], const bf16x8 (&vf)[NB][4],
+                                          f32x16 (&dk)[NB][2], f32x16 (&dv)[NB][2], float c, int half,
+                                          const int (&dbase)[NB], unsigned weff, int row_lim, int krel) {
+    // qsm / gsm: LDS byte addresses of the staged Q and dO tiles; stat_lane: address of this
+    // lane's first lse2 value (rows 4*half..), -delta sits kTile floats further on.
+    // krel (masked variant only): (first key of the wavefront) - (first query position of the
+    // tile); a 32-row block whose rows all precede the keys, or all lost them from their
+    // window, is skipped.
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
+        if (MASKED && ((32 * qb + 31 < krel) || (32 * qb > krel + 32 * NB - 1 + (int)weff - 1) || (32 * qb >= row_lim))) continue;
+        f32x16 s[NB], dp[NB];
+        // phase 1: every LDS read the S / dP MFMAs need is issued before the first MFMA
+        f32x4 nd[4];
+        bf16x8 aq[4], ag[4];
+#pragma unroll
+        for (int a4 = 0; a4 < 4; ++a4) nd[a4] = lds_load128f(stat_lane, (kTile + 32 * qb + 8 * a4) * 4);
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) { aq[ks] = ofrag_nat(qsm, lo, qb, ks); ag[ks] = ofrag_nat(gsm, lo, qb, ks); }
+        GPTOSS_SCHED_FENCE();
+#pragma unroll
+        for (int a4 = 0; a4 < 4; ++a4)
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) { s[nb][4 * a4 + e] = 0.0f; dp[nb][4 * a4 + e] = nd[a4][e]; }
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                s[nb] = mfma_bf16(aq[ks], kf[nb][ks], s[nb]);
+                dp[nb] = mfma_bf16(ag[ks], vf[nb][ks], dp[nb]);
+            }
+        // phase 2: the reads of the second half are issued while those MFMAs run
+        f32x4 lv[4];
+        bf16x8 agt[2][2], aqt[2][2];
+#pragma unroll
+        for (int a4 = 0; a4 < 4; ++a4) lv[a4] = lds_load128f(stat_lane, (32 * qb + 8 * a4) * 4);
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int dblk = 0; dblk < 2; ++dblk) {
+                agt[u][dblk] = ofrag_tr(gsm, lo, qb, u, dblk);
+                aqt[u][dblk] = ofrag_tr(qsm, lo, qb, u, dblk);
+            }
+        GPTOSS_SCHED_FENCE();
+#pragma unroll
+        for (int a4 = 0; a4 < 4; ++a4)
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int i = 4 * a4 + e;
+                    float pe = fast_exp2(fmaf(s[nb][i], c, -lv[a4][e]));
+                    if (MASKED) {
+                        const int r = 32 * qb + 8 * a4 + 4 * half + e;
+                        const bool vis = ((unsigned)(dbase[nb] + r) < weff) & (r < row_lim);
+                        pe = vis ? pe : 0.0f;
+                    }
+                    s[nb][i] = pe;
+                    dp[nb][i] = pe * dp[nb][i];
+                }
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                const bf16x8 pf = cfrag(s[nb], u), dsf = cfrag(dp[nb], u);
+#pragma unroll
+                for (int dblk = 0; dblk < 2; ++dblk) {
+                    dv[nb][dblk] = mfma_bf16(agt[u][dblk], pf, dv[nb][dblk]);
+                    dk[nb][dblk] = mfma_bf16(aqt[u][dblk], dsf, dk[nb][dblk]);
+                }
+            }
+    }
+}
+
+#endif
 template <int NW, int NB>             // NB = 32-key blocks per wavefront
 __global__ __launch_bounds__(NW * 64, (NB == 1 ? 2 : 1)) void attn_bwd_dkdv_kernel(const KArgs a) {
     static_assert(NW == 4, "the asynchronous tile copy is written for 4 wavefronts");

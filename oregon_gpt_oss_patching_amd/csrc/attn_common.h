@@ -64,6 +64,10 @@ __device__ __forceinline__ bf16x8 as_bf16x8(const u32x4 v) {
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+// max(a, b) as median(a, b, +inf): one v_med3_f32, without the NaN-quieting pre-pass that
+// fmaxf costs in IEEE mode (the kernels never produce NaN: masked logits are -inf and the
+// running max is finite).
+__device__ __forceinline__ float fast_max(float a, float b) { return __builtin_amdgcn_fmed3f(a, b, INFINITY); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
 // ---- staging a 64 x 64 tile: global -> registers -> LDS, NT threads --------------

@@ -68,11 +68,13 @@ __device__ __forceinline__ void fwd_tile(uint32_t ksm, uint32_t vsm, const TileL
                     }
                 }
         }
-        float mx = fmaxf(s[0][qb][0], s[1][qb][0]);
+        // two independent reduction chains keep the VALU pipelined
+        float mx0 = s[0][qb][0], mx1 = s[1][qb][0];
 #pragma unroll
-        for (int i = 1; i < 16; ++i) mx = fmaxf(mx, fmaxf(s[0][qb][i], s[1][qb][i]));
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float m_new = fmaxf(m[qb], mx * c);
+        for (int i = 1; i < 16; ++i) { mx0 = fast_max(mx0, s[0][qb][i]); mx1 = fast_max(mx1, s[1][qb][i]); }
+        float mx = fast_max(mx0, mx1);
+        mx = fast_max(mx, __shfl_xor(mx, 32));
+        const float m_new = fast_max(m[qb], mx * c);
         if (__builtin_amdgcn_ballot_w64(m_new != m[qb]) != 0ull) {
             const float alpha = fast_exp2(m[qb] - m_new);
             l[qb] *= alpha;
