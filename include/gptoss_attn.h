@@ -32,6 +32,12 @@
  *   seqlens      (B,) int32 or NULL: right-padding lengths.  Keys at or beyond
  *                seqlens[b] are invisible; query rows at or beyond it produce
  *                O = 0, lse = sink and contribute no gradient.
+ *   doc_start    (B, Sq) int32 or NULL, for rows packed from several documents:
+ *                doc_start[b][i] is the index of the first token of the document
+ *                that query i belongs to (non-decreasing along i); keys before it
+ *                are invisible.  Needs Sq == Skv and q_offset == 0.  NULL (what
+ *                the reference does, it ignores position ids) lets documents of a
+ *                packed row see each other.
  * Visibility of key j to the query at absolute position p = q_offset + i:
  *   j <= p  and  (window == 0 or j > p - window)      (attention_kernel.py:68,71)
  */
@@ -45,7 +51,7 @@
 extern "C" {
 #endif
 
-#define GPTOSS_ATTN_ABI_VERSION 1
+#define GPTOSS_ATTN_ABI_VERSION 2
 
 enum gptoss_attn_dtype {
     GPTOSS_ATTN_BF16 = 0, /* 2-byte bfloat16 tensors, fp32 accumulation */
@@ -58,7 +64,8 @@ enum gptoss_attn_status {
     GPTOSS_ATTN_ERR_NULL_TENSOR = -2,   /* a required tensor pointer is NULL */
     GPTOSS_ATTN_ERR_HEAD_DIM = -3,      /* D != 64 */
     GPTOSS_ATTN_ERR_HEADS = -4,         /* H <= 0, G <= 0 or H % G != 0 */
-    GPTOSS_ATTN_ERR_SHAPE = -5,         /* B, Sq or Skv <= 0, window < 0, q_offset < 0 */
+    GPTOSS_ATTN_ERR_SHAPE = -5,         /* B, Sq or Skv <= 0, window < 0, q_offset < 0, scale <= 0,
+                                           or doc_start with Sq != Skv or q_offset != 0 */
     GPTOSS_ATTN_ERR_DTYPE = -6,         /* dtype not in gptoss_attn_dtype */
     GPTOSS_ATTN_ERR_ALIGNMENT = -7,     /* a tensor base or stride breaks 16-byte row alignment */
     GPTOSS_ATTN_ERR_STRIDE = -8,        /* a sequence stride smaller than D */
@@ -83,6 +90,7 @@ typedef struct gptoss_attn_params {
     const void *q, *k, *v;
     const float *sinks;     /* optional */
     const int32_t *seqlens; /* optional */
+    const int32_t *doc_start; /* optional */
     void *o;
     float *lse;
 
@@ -105,7 +113,7 @@ const char *gptoss_attn_status_string(int status);
  * Forward: O and logsumexp.  Replaces the `_attn_fwd` launch in
  * `_attention.forward` (attention_kernel.py:11-100, 241-262) including the
  * output transpose copy at :272 (O is written directly in the caller's layout).
- * Reads q,k,v,sinks,seqlens; writes o,lse.
+ * Reads q,k,v,sinks,seqlens,doc_start; writes o,lse.
  */
 int gptoss_attn_fwd(const gptoss_attn_params *params, void *stream);
 
@@ -122,13 +130,13 @@ int gptoss_attn_bwd_preprocess(const gptoss_attn_params *params, void *stream);
 /*
  * Backward step 2: dK and dV, KV-outer, no atomics (deterministic).  Replaces
  * the dv/dk halves of `_attn_bwd` (attention_kernel.py:199-212).
- * Reads q,k,v,d_o,lse,delta,seqlens; writes dk,dv.
+ * Reads q,k,v,d_o,lse,delta,seqlens,doc_start; writes dk,dv.
  */
 int gptoss_attn_bwd_dkdv(const gptoss_attn_params *params, void *stream);
 
 /*
  * Backward step 3: dQ.  Replaces the dq half of `_attn_bwd`
- * (attention_kernel.py:206-217).  Reads q,k,v,d_o,lse,delta,seqlens; writes dq.
+ * (attention_kernel.py:206-217).  Reads q,k,v,d_o,lse,delta,seqlens,doc_start; writes dq.
  */
 int gptoss_attn_bwd_dq(const gptoss_attn_params *params, void *stream);
 

@@ -30,6 +30,8 @@
  *   - `seqlens` (right padding) is an addition: keys >= len are masked like
  *     too-old keys, and query rows >= len see no key at all.
  *   - start_q (:44-47) is taken by value as q_offset.
+ *   - `doc_start` (packed rows) is an addition: keys before the first token of the
+ *     query's own document are masked.
  *
  * Pinning: tests/test_oracle_tiled.py checks every function here against
  * eager_ref.py (itself pinned by golden vectors and closed forms).
@@ -45,19 +47,21 @@
 static inline int imax(int a, int b) { return a > b ? a : b; }
 static inline int imin(int a, int b) { return a < b ? a : b; }
 
-/* 1 when key j is hidden from the query at absolute position pos. */
-static inline int masked(int j, int pos, int window, int len)
+/* 1 when key j is hidden from the query at absolute position pos; `first` is the
+   first key of the query's own document (0 unless rows are packed). */
+static inline int masked(int j, int pos, int window, int len, int first)
 {
     if (j > pos) return 1;                          /* :68  */
     if (window > 0 && j < pos - window + 1) return 1; /* :71  */
     if (j >= len || pos >= len) return 1;           /* right padding */
+    if (j < first) return 1;                        /* another document of a packed row */
     return 0;
 }
 
 int oracle_attn_fwd(const float *q, const float *k, const float *v, const float *sinks,
                     float *o, float *lse,
                     int B, int H, int G, int Sq, int Skv, int D,
-                    float scale, int window, int q_offset, const int *seqlens)
+                    float scale, int window, int q_offset, const int *seqlens, const int *doc_start)
 {
     if (!q || !k || !v || !o || !lse || G <= 0 || H % G) return -1;
     const int r = H / G;
@@ -81,12 +85,13 @@ int oracle_attn_fwd(const float *q, const float *k, const float *v, const float 
                 const int cols = imin(TILE, Skv - n0);
                 for (int i = 0; i < rows; ++i) {
                     const int pos = q_offset + m0 + i;
+                    const int first = doc_start ? doc_start[(size_t)b * Sq + m0 + i] : 0;
                     const float *qi = q + (((size_t)b * H + h) * Sq + m0 + i) * D;
                     double mx = m_i[i];
                     for (int j = 0; j < cols; ++j) {
                         double dot = 0.0;
                         for (int d = 0; d < D; ++d) dot += (double)qi[d] * (double)kb[(size_t)(n0 + j) * D + d];
-                        s[j] = dot * scale + (masked(n0 + j, pos, window, len) ? MASK_ADD : 0.0);
+                        s[j] = dot * scale + (masked(n0 + j, pos, window, len, first) ? MASK_ADD : 0.0);
                         if (s[j] > mx) mx = s[j];
                     }
                     const double alpha = exp(m_i[i] - mx);
@@ -135,7 +140,7 @@ int oracle_attn_bwd(const float *q, const float *k, const float *v, const float 
                     const float *lse, const float *delta, const float *d_o,
                     float *dq, float *dk, float *dv, float *dsinks,
                     int B, int H, int G, int Sq, int Skv, int D,
-                    float scale, int window, int q_offset, const int *seqlens)
+                    float scale, int window, int q_offset, const int *seqlens, const int *doc_start)
 {
     if (!q || !k || !v || !lse || !delta || !d_o || !dq || !dk || !dv || G <= 0 || H % G) return -1;
     const int r = H / G;
@@ -160,6 +165,7 @@ int oracle_attn_bwd(const float *q, const float *k, const float *v, const float 
                 if (window > 0) lo = imax(0, q_offset + m0 - window);
                 for (int i = 0; i < rows; ++i) {
                     const int pos = q_offset + m0 + i;
+                    const int first = doc_start ? doc_start[(size_t)b * Sq + m0 + i] : 0;
                     const size_t row = ((size_t)b * H + h) * Sq + m0 + i;
                     const float *qi = q + row * D;
                     const float *gi = d_o + (((size_t)b * Sq + m0 + i) * H + h) * D;
@@ -175,7 +181,7 @@ int oracle_attn_bwd(const float *q, const float *k, const float *v, const float 
                                 dot += (double)qi[d] * (double)kj[d];
                                 dp += (double)gi[d] * (double)vj[d];
                             }
-                            const double sij = dot * scale + (masked(n0 + j, pos, window, len) ? MASK_ADD : 0.0);
+                            const double sij = dot * scale + (masked(n0 + j, pos, window, len, first) ? MASK_ADD : 0.0);
                             const double p = exp(sij - Mi);       /* :199 */
                             const double ds = p * (dp - Di);       /* :207 */
                             double *dkj = dkb + (size_t)(n0 + j) * D;

@@ -43,6 +43,7 @@ def allowed_mask(
     q_offset: int = 0,
     seqlens: Optional[Sequence[int]] = None,
     batch: int = 1,
+    doc_start: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """Boolean (B, 1, Sq, Skv) mask, True where query row i may see key j.
 
@@ -52,7 +53,10 @@ def allowed_mask(
     full-causal layer, which is how the reference treats a falsy BANDWIDTH
     (attention_kernel.py:60-63).  With ``seqlens`` (right padding), keys at or
     beyond the row's valid length are hidden and so is every key for a padded
-    query row.
+    query row.  With ``doc_start`` (B, Sq) -- for packed rows, the index of the
+    first token of the document each query belongs to -- keys before it are
+    hidden, which for a causal mask is exactly transformers' same-document
+    predicate (masking_utils.py:182-190).
     """
     i = torch.arange(sq).view(sq, 1) + q_offset
     j = torch.arange(skv).view(1, skv)
@@ -65,6 +69,9 @@ def allowed_mask(
         kvalid = torch.arange(skv).view(1, 1, 1, skv) < lens
         qvalid = (torch.arange(sq).view(1, 1, sq, 1) + q_offset) < lens
         ok = ok & kvalid & qvalid
+    if doc_start is not None:
+        ds = torch.as_tensor(doc_start).to(torch.long).view(batch, 1, sq, 1)
+        ok = ok & (torch.arange(skv).view(1, 1, 1, skv) >= ds)
     return ok
 
 
@@ -83,6 +90,7 @@ def eager_attention(
     window: Optional[int] = None,
     q_offset: int = 0,
     seqlens: Optional[Sequence[int]] = None,
+    doc_start: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """Eager attention with a sink column; returns (B, Sq, H, D).
 
@@ -100,7 +108,7 @@ def eager_attention(
     kk = repeat_kv(k, r)
     vv = repeat_kv(v, r)
     logits = torch.matmul(q, kk.transpose(2, 3)) * scale
-    ok = allowed_mask(sq, skv, window, q_offset, seqlens, b).to(q.device)
+    ok = allowed_mask(sq, skv, window, q_offset, seqlens, b, doc_start).to(q.device)
     logits = logits.masked_fill(~ok, float("-inf"))
     if sinks is None:
         sink_col = torch.zeros(1, h, 1, 1, dtype=q.dtype, device=q.device)
@@ -121,6 +129,7 @@ def logsumexp_rows(
     window: Optional[int] = None,
     q_offset: int = 0,
     seqlens: Optional[Sequence[int]] = None,
+    doc_start: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """(B, H, Sq) natural-log logsumexp over the visible logits and the sink,
     the quantity the reference stores as M (attention_kernel.py:93-98)."""
@@ -128,7 +137,7 @@ def logsumexp_rows(
     g, skv = k.shape[1], k.shape[2]
     kk = repeat_kv(k, h // g)
     logits = torch.matmul(q, kk.transpose(2, 3)) * scale
-    ok = allowed_mask(sq, skv, window, q_offset, seqlens, b).to(q.device)
+    ok = allowed_mask(sq, skv, window, q_offset, seqlens, b, doc_start).to(q.device)
     logits = logits.masked_fill(~ok, float("-inf"))
     if sinks is None:
         sink_col = torch.zeros(1, h, 1, 1, dtype=q.dtype, device=q.device)
@@ -148,6 +157,7 @@ def eager_attention_grads(
     window: Optional[int] = None,
     q_offset: int = 0,
     seqlens: Optional[Sequence[int]] = None,
+    doc_start: Optional[torch.Tensor] = None,
 ):
     """Forward + autograd backward.  ``d_out`` is (B, Sq, H, D), the layout in
     which the gradient reaches the op (attention_kernel.py:290).  Returns
@@ -156,7 +166,7 @@ def eager_attention_grads(
     k = k.detach().clone().requires_grad_(True)
     v = v.detach().clone().requires_grad_(True)
     s = sinks.detach().clone().requires_grad_(True)
-    out = eager_attention(q, k, v, s, scale, window, q_offset, seqlens)
+    out = eager_attention(q, k, v, s, scale, window, q_offset, seqlens, doc_start)
     dq, dk, dv, ds = torch.autograd.grad(out, (q, k, v, s), d_out)
     return out.detach(), dq, dk, dv, ds
 
@@ -197,3 +207,17 @@ def attention_flops(b: int, h: int, d: int, pairs: int):
     """Algorithmic FLOPs: 2 GEMMs forward, 5 backward, 2*D flops per pair each."""
     unit = 2 * d * pairs * b * h
     return {"fwd": 2 * unit, "bwd": 5 * unit, "total": 7 * unit}
+
+
+def doc_start_from_lengths(doc_lens: Sequence[Sequence[int]], s: int) -> torch.Tensor:
+    """(B, S) int32 document-start index per token for rows packed from documents of the
+    given lengths (each row's lengths must sum to ``s``)."""
+    rows = []
+    for lens in doc_lens:
+        assert sum(lens) == s
+        starts, pos = [], 0
+        for n in lens:
+            starts += [pos] * n
+            pos += n
+        rows.append(starts)
+    return torch.tensor(rows, dtype=torch.int32)

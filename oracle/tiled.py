@@ -47,7 +47,7 @@ def _ip(seqlens: Optional[Sequence[int]]):
     return arr, ctypes.cast(arr, ctypes.c_void_p)
 
 
-def tiled_fwd(q, k, v, sinks, scale, window=None, q_offset=0, seqlens=None):
+def tiled_fwd(q, k, v, sinks, scale, window=None, q_offset=0, seqlens=None, doc_start=None):
     """q (B,H,Sq,D), k/v (B,G,Skv,D) fp32 -> (o (B,Sq,H,D), lse (B,H,Sq))."""
     q, k, v = (t.detach().float().contiguous() for t in (q, k, v))
     s = None if sinks is None else sinks.detach().float().contiguous()
@@ -56,15 +56,16 @@ def tiled_fwd(q, k, v, sinks, scale, window=None, q_offset=0, seqlens=None):
     o = torch.empty(b, sq, h, d)
     lse = torch.empty(b, h, sq)
     keep, sl = _ip(seqlens)
+    keep2, dsp = _ip(None if doc_start is None else torch.as_tensor(doc_start).reshape(-1).tolist())
     rc = lib().oracle_attn_fwd(_fp(q), _fp(k), _fp(v), _fp(s), _fp(o), _fp(lse),
                                b, h, g, sq, skv, d, ctypes.c_float(scale),
-                               int(window or 0), int(q_offset), sl)
+                               int(window or 0), int(q_offset), sl, dsp)
     if rc:
         raise RuntimeError(f"oracle_attn_fwd rc={rc}")
     return o, lse
 
 
-def tiled_bwd(q, k, v, sinks, o, lse, d_o, scale, window=None, q_offset=0, seqlens=None):
+def tiled_bwd(q, k, v, sinks, o, lse, d_o, scale, window=None, q_offset=0, seqlens=None, doc_start=None):
     """Returns (dq, dk, dv, dsinks, delta); o and d_o are (B,Sq,H,D)."""
     q, k, v, o, lse, d_o = (t.detach().float().contiguous() for t in (q, k, v, o, lse, d_o))
     s = None if sinks is None else sinks.detach().float().contiguous()
@@ -77,10 +78,11 @@ def tiled_bwd(q, k, v, sinks, o, lse, d_o, scale, window=None, q_offset=0, seqle
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     dsinks = torch.empty(h)
     keep, sl = _ip(seqlens)
+    keep2, dsp = _ip(None if doc_start is None else torch.as_tensor(doc_start).reshape(-1).tolist())
     rc = lib().oracle_attn_bwd(_fp(q), _fp(k), _fp(v), _fp(s), _fp(lse), _fp(delta), _fp(d_o),
                                _fp(dq), _fp(dk), _fp(dv), _fp(dsinks),
                                b, h, g, sq, skv, d, ctypes.c_float(scale),
-                               int(window or 0), int(q_offset), sl)
+                               int(window or 0), int(q_offset), sl, dsp)
     if rc:
         raise RuntimeError(f"oracle_attn_bwd rc={rc}")
     return dq, dk, dv, dsinks, delta

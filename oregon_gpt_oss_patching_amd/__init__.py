@@ -8,9 +8,10 @@ from .attention_kernel import (  # noqa: F401
     attention,
     attention_backward,
     attention_forward,
+    doc_start_from_position_ids,
     hip_flash_attention,
     triton_flash_attention,
 )
 
-__all__ = ["attention", "attention_forward", "attention_backward", "hip_flash_attention",
-           "triton_flash_attention"]
+__all__ = ["attention", "attention_forward", "attention_backward", "doc_start_from_position_ids",
+           "hip_flash_attention", "triton_flash_attention"]

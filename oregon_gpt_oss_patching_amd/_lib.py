@@ -12,7 +12,7 @@ from typing import Optional
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIBRARY = os.path.join(_HERE, "libgptoss_attn.so")
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 DTYPE_BF16 = 0
 DTYPE_FP32 = 1
 
@@ -47,6 +47,7 @@ class Params(ctypes.Structure):
         ("q", ctypes.c_void_p), ("k", ctypes.c_void_p), ("v", ctypes.c_void_p),
         ("sinks", ctypes.c_void_p),
         ("seqlens", ctypes.c_void_p),
+        ("doc_start", ctypes.c_void_p),
         ("o", ctypes.c_void_p),
         ("lse", ctypes.c_void_p),
         ("d_o", ctypes.c_void_p),

@@ -27,9 +27,14 @@ import torch
 
 from . import _lib
 
-__all__ = ["attention", "triton_flash_attention", "hip_flash_attention", "attention_forward", "attention_backward"]
+__all__ = ["attention", "triton_flash_attention", "hip_flash_attention", "attention_forward", "attention_backward",
+           "doc_start_from_position_ids"]
 
 _DTYPES = {torch.bfloat16: _lib.DTYPE_BF16}
+
+# When True the Hugging Face adapter masks across documents of packed rows (from the
+# `position_ids` it is handed).  False reproduces the reference, which ignores position ids.
+RESPECT_PACKING = False
 
 
 def _strides_bhs(t: torch.Tensor, layout: str):
@@ -64,7 +69,7 @@ def _check_inputs(q, k, v, sinks):
         raise RuntimeError("sinks must hold one logit per query head")
 
 
-def _base_params(q, k, v, sinks32, seqlens, scale, window, q_offset):
+def _base_params(q, k, v, sinks32, seqlens, scale, window, q_offset, doc_start=None):
     p = _lib.new_params()
     b, h, sq, d = q.shape
     g, skv = k.shape[1], k.shape[2]
@@ -76,6 +81,7 @@ def _base_params(q, k, v, sinks32, seqlens, scale, window, q_offset):
     p.q, p.k, p.v = q.data_ptr(), k.data_ptr(), v.data_ptr()
     p.sinks = sinks32.data_ptr() if sinks32 is not None else None
     p.seqlens = seqlens.data_ptr() if seqlens is not None else None
+    p.doc_start = doc_start.data_ptr() if doc_start is not None else None
     _set(p.q_stride, _strides_bhs(q, "bhsd"))
     _set(p.k_stride, _strides_bhs(k, "bhsd"))
     _set(p.v_stride, _strides_bhs(v, "bhsd"))
@@ -95,17 +101,40 @@ def _prep_seqlens(seqlens, device, batch):
     return sl
 
 
-def attention_forward(q, k, v, sinks, sm_scale, window=None, q_offset=0, seqlens=None):
+def _prep_doc_start(doc_start, q):
+    if doc_start is None:
+        return None
+    ds = torch.as_tensor(doc_start, device=q.device).to(torch.int32).contiguous()
+    if ds.shape != (q.shape[0], q.shape[2]):
+        raise RuntimeError("doc_start must be (B, S): the first token index of each query's document")
+    return ds
+
+
+def doc_start_from_position_ids(position_ids: torch.Tensor) -> torch.Tensor:
+    """(B, S) int32 document-start index per token of packed rows, from position ids that restart
+    at every document (the convention transformers detects packing by, masking_utils.py:728-757):
+    a new document begins wherever the position does not follow its predecessor by one."""
+    pos = position_ids
+    b, s = pos.shape
+    idx = torch.arange(s, device=pos.device).view(1, s).expand(b, s)
+    new_doc = torch.ones_like(pos, dtype=torch.bool)
+    new_doc[:, 1:] = (pos[:, 1:] - pos[:, :-1]) != 1
+    starts = torch.where(new_doc, idx, torch.zeros_like(idx))
+    return torch.cummax(starts, dim=1).values.to(torch.int32)
+
+
+def attention_forward(q, k, v, sinks, sm_scale, window=None, q_offset=0, seqlens=None, doc_start=None):
     """Runs the forward kernel.  Returns (o (B,S,H,D), lse (B,H,S) fp32)."""
     _check_inputs(q, k, v, sinks)
     q, k, v = _row_contiguous(q), _row_contiguous(k), _row_contiguous(v)
     b, h, sq, d = q.shape
     sinks32 = None if sinks is None else sinks.detach().to(torch.float32).contiguous()
     sl = _prep_seqlens(seqlens, q.device, b)
+    ds = _prep_doc_start(doc_start, q)
     o = torch.empty((b, sq, h, d), dtype=q.dtype, device=q.device)
     lse = torch.empty((b, h, sq), dtype=torch.float32, device=q.device)
     with torch.cuda.device(q.device):
-        p = _base_params(q, k, v, sinks32, sl, sm_scale, window, q_offset)
+        p = _base_params(q, k, v, sinks32, sl, sm_scale, window, q_offset, ds)
         p.o, p.lse = o.data_ptr(), lse.data_ptr()
         _set(p.o_stride, _strides_bhs(o, "bshd"))
         _lib.call("gptoss_attn_fwd", p, _stream(q))
@@ -113,7 +142,7 @@ def attention_forward(q, k, v, sinks, sm_scale, window=None, q_offset=0, seqlens
 
 
 def attention_backward(q, k, v, sinks, o, lse, d_o, sm_scale, window=None, q_offset=0, seqlens=None,
-                       need_dsinks=True):
+                       need_dsinks=True, doc_start=None):
     """Runs the three backward kernels.  o and d_o are (B,S,H,D).
     Returns (dq, dk, dv, dsinks_fp32_or_None)."""
     _check_inputs(q, k, v, sinks)
@@ -122,13 +151,14 @@ def attention_backward(q, k, v, sinks, o, lse, d_o, sm_scale, window=None, q_off
     b, h, sq, d = q.shape
     sinks32 = None if sinks is None else sinks.detach().to(torch.float32).contiguous()
     sl = _prep_seqlens(seqlens, q.device, b)
+    ds = _prep_doc_start(doc_start, q)
     dq = torch.empty((b, h, sq, d), dtype=q.dtype, device=q.device)
     dk = torch.empty(k.shape, dtype=k.dtype, device=q.device)
     dv = torch.empty(v.shape, dtype=v.dtype, device=q.device)
     delta = torch.empty((2, b, h, sq), dtype=torch.float32, device=q.device)   # [delta; lse*log2e]
     dsinks = torch.empty((h,), dtype=torch.float32, device=q.device) if need_dsinks else None
     with torch.cuda.device(q.device):
-        p = _base_params(q, k, v, sinks32, sl, sm_scale, window, q_offset)
+        p = _base_params(q, k, v, sinks32, sl, sm_scale, window, q_offset, ds)
         p.o, p.lse = o.data_ptr(), lse.data_ptr()
         _set(p.o_stride, _strides_bhs(o, "bshd"))
         p.d_o = d_o.data_ptr()
@@ -145,31 +175,42 @@ def attention_backward(q, k, v, sinks, o, lse, d_o, sm_scale, window=None, q_off
 
 class _attention(torch.autograd.Function):
     """Same argument list and gradient tuple as the reference's `_attention`
-    (attention_kernel.py:220-344), plus an optional trailing `seqlens`."""
+    (attention_kernel.py:220-344), plus optional trailing `seqlens` and `doc_start`.
+
+    The kernels compute on bfloat16 tensors.  float32 / float16 tensors are accepted for
+    convenience (the reference runs them natively): they are rounded to bfloat16 on the
+    way in and the results cast back, so their accuracy is bfloat16's, not float32's."""
 
     @staticmethod
-    def forward(ctx, q, k, v, sinks, sm_scale, bandwidth, start_q, seqlens=None):
+    def forward(ctx, q, k, v, sinks, sm_scale, bandwidth, start_q, seqlens=None, doc_start=None):
+        ctx.in_dtypes = (q.dtype, k.dtype, v.dtype)
+        if q.dtype in (torch.float32, torch.float16):
+            q, k, v = (t.to(torch.bfloat16) for t in (q, k, v))
         q_offset = 0
         if start_q is not None:
             q_offset = int(start_q.item()) if torch.is_tensor(start_q) else int(start_q)
-        o, lse = attention_forward(q, k, v, sinks, sm_scale, bandwidth, q_offset, seqlens)
-        ctx.save_for_backward(q, k, v, sinks, o, lse, seqlens if torch.is_tensor(seqlens) else None)
+        if doc_start is not None:
+            doc_start = _prep_doc_start(doc_start, q)
+        o, lse = attention_forward(q, k, v, sinks, sm_scale, bandwidth, q_offset, seqlens, doc_start)
+        ctx.save_for_backward(q, k, v, sinks, o, lse, seqlens if torch.is_tensor(seqlens) else None, doc_start)
         ctx.seqlens_list = None if torch.is_tensor(seqlens) else seqlens
         ctx.sm_scale = sm_scale
         ctx.bandwidth = bandwidth
         ctx.q_offset = q_offset
-        return o
+        return o.to(ctx.in_dtypes[0])
 
     @staticmethod
     def backward(ctx, do):
-        q, k, v, sinks, o, lse, seqlens_t = ctx.saved_tensors
+        q, k, v, sinks, o, lse, seqlens_t, doc_start = ctx.saved_tensors
         seqlens = seqlens_t if seqlens_t is not None else ctx.seqlens_list
         need_ds = sinks is not None and ctx.needs_input_grad[3]
         dq, dk, dv, dsinks = attention_backward(
-            q, k, v, sinks, o, lse, do, ctx.sm_scale, ctx.bandwidth, ctx.q_offset, seqlens, need_dsinks=need_ds)
+            q, k, v, sinks, o, lse, do.to(q.dtype), ctx.sm_scale, ctx.bandwidth, ctx.q_offset, seqlens,
+            need_dsinks=need_ds, doc_start=doc_start)
         if dsinks is not None:
             dsinks = dsinks.to(sinks.dtype).view_as(sinks)
-        return dq, dk, dv, dsinks, None, None, None, None
+        qd, kd, vd = ctx.in_dtypes
+        return dq.to(qd), dk.to(kd), dv.to(vd), dsinks, None, None, None, None, None
 
 
 attention = _attention.apply
@@ -190,13 +231,22 @@ def hip_flash_attention(
     Like the reference it ignores `attention_mask` and `dropout`: causality and the
     sliding window come from `module.sliding_window`, the sink logits from
     `module.sinks`.  A caller with right-padded batches may pass `seqlens=` in
-    kwargs, or hand a 1-D integer tensor of valid lengths over as `attention_mask`."""
+    kwargs, or hand a 1-D integer tensor of valid lengths over as `attention_mask`.  Rows
+    packed from several documents attend across documents, as in the reference, unless the
+    caller passes `doc_start=` (see `doc_start_from_position_ids`) or packing awareness was
+    switched on with `patch_flash_attention(respect_packing=True)`, in which case the
+    `position_ids` the model passes along are used."""
+    doc_start = kwargs.get("doc_start")
+    if doc_start is None and RESPECT_PACKING and kwargs.get("position_ids") is not None:
+        pos = kwargs["position_ids"]
+        if pos.dim() == 2 and pos.shape[0] == query.shape[0] and pos.shape[1] == query.shape[2] == key.shape[2]:
+            doc_start = doc_start_from_position_ids(pos)
     seqlens = kwargs.get("seqlens")
     if (seqlens is None and torch.is_tensor(attention_mask) and attention_mask.dim() == 1
             and not attention_mask.dtype.is_floating_point):
         # valid lengths handed over in place of the dense mask (see sft_bench.mask_free_attention_mask)
         seqlens = attention_mask
-    out = attention(query, key, value, module.sinks, scaling, module.sliding_window, None, seqlens)
+    out = attention(query, key, value, module.sinks, scaling, module.sliding_window, None, seqlens, doc_start)
     return out, None
 
 

@@ -102,14 +102,16 @@ __global__ __launch_bounds__(1024) void attn_bwd_dsinks_kernel(const KArgs a) {
 // lane's key), or a huge negative number for a dead key, so that pair (row r, key)
 // is visible iff 0 <= dbase + r < weff, tested with one unsigned compare; rows at
 // or beyond `row_lim` (relative to the tile) do not exist.
-#ifndef GPTOSS_DKDV_PIPE
-template <bool MASKED, int NB>
+template <bool MASKED, bool DOCS, int NB>
 __device__ __forceinline__ void dkdv_tile(uint32_t qsm, uint32_t gsm, uint32_t stat_lane, const TileLaneOffsets &lo,
                                           const bf16x8 (&kf)[NB][4], const bf16x8 (&vf)[NB][4],
                                           f32x16 (&dk)[NB][2], f32x16 (&dv)[NB][2], float c, int half,
-                                          const int (&dbase)[NB], unsigned weff, int row_lim, int krel) {
+                                          const int (&dbase)[NB], unsigned weff, int row_lim, int krel,
+                                          uint32_t ds_lane, const int (&jkey)[NB]) {
     // qsm / gsm: LDS byte addresses of the staged Q and dO tiles; stat_lane: address of this
     // lane's first lse2 value (rows 4*half..), -delta sits kTile floats further on.
+    // DOCS (packed rows): ds_lane addresses the staged document starts of the same rows, jkey
+    // is the lane's key index; a key before its query's document start is invisible.
     // krel (masked variant only): (first key of the wavefront) - (first query position of the
     // tile); a 32-row block whose rows all precede the keys, or all lost them from their
     // window, is skipped.
@@ -139,6 +141,8 @@ __device__ __forceinline__ void dkdv_tile(uint32_t qsm, uint32_t gsm, uint32_t s
 #pragma unroll
         for (int a4 = 0; a4 < 4; ++a4) {
             const f32x4 lv = lds_load128f(stat_lane, (32 * qb + 8 * a4) * 4);
+            u32x4 dsr = {0u, 0u, 0u, 0u};
+            if (MASKED && DOCS) dsr = lds_load128(ds_lane, (32 * qb + 8 * a4) * 4);
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
@@ -147,7 +151,8 @@ __device__ __forceinline__ void dkdv_tile(uint32_t qsm, uint32_t gsm, uint32_t s
                     float pe = fast_exp2(fmaf(s[nb][i], c, -lv[e]));
                     if (MASKED) {
                         const int r = 32 * qb + 8 * a4 + 4 * half + e;
-                        const bool vis = ((unsigned)(dbase[nb] + r) < weff) & (r < row_lim);
+                        bool vis = ((unsigned)(dbase[nb] + r) < weff) & (r < row_lim);
+                        if (DOCS) vis = vis & (jkey[nb] >= (int)dsr[e]);
                         pe = vis ? pe : 0.0f;
                     }
                     s[nb][i] = pe;
@@ -175,87 +180,7 @@ __device__ __forceinline__ void dkdv_tile(uint32_t qsm, uint32_t gsm, uint32_t s
     }
 }
 
-#else
-template <bool MASKED, int NB>
-__device__ __forceinline__ void dkdv_tile(uint32_t qsm, uint32_t gsm, uint32_t stat_lane, const TileLaneOffsets &lo,
-                                          const bf16x8 (&kf)[NB][4], const bf16x8 (&vf)[NB][4],
-                                          f32x16 (&dk)[NB][2], f32x16 (&dv)[NB][2], float c, int half,
-                                          const int (&dbase)[NB], unsigned weff, int row_lim, int krel) {
-    // qsm / gsm: LDS byte addresses of the staged Q and dO tiles; stat_lane: address of this
-    // lane's first lse2 value (rows 4*half..), -delta sits kTile floats further on.
-    // krel (masked variant only): (first key of the wavefront) - (first query position of the
-    // tile); a 32-row block whose rows all precede the keys, or all lost them from their
-    // window, is skipped.
-#pragma unroll
-    for (int qb = 0; qb < 2; ++qb) {
-        if (MASKED && ((32 * qb + 31 < krel) || (32 * qb > krel + 32 * NB - 1 + (int)weff - 1) || (32 * qb >= row_lim))) continue;
-        f32x16 s[NB], dp[NB];
-        // phase 1: every LDS read the S / dP MFMAs need is issued before the first MFMA
-        f32x4 nd[4];
-        bf16x8 aq[4], ag[4];
-#pragma unroll
-        for (int a4 = 0; a4 < 4; ++a4) nd[a4] = lds_load128f(stat_lane, (kTile + 32 * qb + 8 * a4) * 4);
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks) { aq[ks] = ofrag_nat(qsm, lo, qb, ks); ag[ks] = ofrag_nat(gsm, lo, qb, ks); }
-        GPTOSS_SCHED_FENCE();
-#pragma unroll
-        for (int a4 = 0; a4 < 4; ++a4)
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-                for (int e = 0; e < 4; ++e) { s[nb][4 * a4 + e] = 0.0f; dp[nb][4 * a4 + e] = nd[a4][e]; }
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb) {
-                s[nb] = mfma_bf16(aq[ks], kf[nb][ks], s[nb]);
-                dp[nb] = mfma_bf16(ag[ks], vf[nb][ks], dp[nb]);
-            }
-        // phase 2: the reads of the second half are issued while those MFMAs run
-        f32x4 lv[4];
-        bf16x8 agt[2][2], aqt[2][2];
-#pragma unroll
-        for (int a4 = 0; a4 < 4; ++a4) lv[a4] = lds_load128f(stat_lane, (32 * qb + 8 * a4) * 4);
-#pragma unroll
-        for (int u = 0; u < 2; ++u)
-#pragma unroll
-            for (int dblk = 0; dblk < 2; ++dblk) {
-                agt[u][dblk] = ofrag_tr(gsm, lo, qb, u, dblk);
-                aqt[u][dblk] = ofrag_tr(qsm, lo, qb, u, dblk);
-            }
-        GPTOSS_SCHED_FENCE();
-#pragma unroll
-        for (int a4 = 0; a4 < 4; ++a4)
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb)
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int i = 4 * a4 + e;
-                    float pe = fast_exp2(fmaf(s[nb][i], c, -lv[a4][e]));
-                    if (MASKED) {
-                        const int r = 32 * qb + 8 * a4 + 4 * half + e;
-                        const bool vis = ((unsigned)(dbase[nb] + r) < weff) & (r < row_lim);
-                        pe = vis ? pe : 0.0f;
-                    }
-                    s[nb][i] = pe;
-                    dp[nb][i] = pe * dp[nb][i];
-                }
-#pragma unroll
-        for (int u = 0; u < 2; ++u)
-#pragma unroll
-            for (int nb = 0; nb < NB; ++nb) {
-                const bf16x8 pf = cfrag(s[nb], u), dsf = cfrag(dp[nb], u);
-#pragma unroll
-                for (int dblk = 0; dblk < 2; ++dblk) {
-                    dv[nb][dblk] = mfma_bf16(agt[u][dblk], pf, dv[nb][dblk]);
-                    dk[nb][dblk] = mfma_bf16(aqt[u][dblk], dsf, dk[nb][dblk]);
-                }
-            }
-    }
-}
-
-#endif
-template <int NW, int NB>             // NB = 32-key blocks per wavefront
+template <int NW, int NB, bool DOCS>  // NB = 32-key blocks per wavefront; DOCS = packed rows (doc_start given)
 __global__ __launch_bounds__(NW * 64, (NB == 1 ? 2 : 1)) void attn_bwd_dkdv_kernel(const KArgs a) {
     static_assert(NW == 4, "the asynchronous tile copy is written for 4 wavefronts");
     constexpr int NS = 3;              // LDS stages: tiles are requested two iterations ahead
@@ -263,6 +188,7 @@ __global__ __launch_bounds__(NW * 64, (NB == 1 ? 2 : 1)) void attn_bwd_dkdv_kern
     constexpr int BN = WK * NW;        // keys per workgroup
     __shared__ __attribute__((aligned(16))) char smem[NS][2][kStageTileBytes];
     __shared__ __attribute__((aligned(16))) float sstat[NS][2][kTile];
+    __shared__ __attribute__((aligned(16))) int32_t sdoc[DOCS ? NS : 1][kTile];   // document starts of the staged rows
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int l32 = lane & 31, half = lane >> 5;
@@ -321,6 +247,11 @@ __global__ __launch_bounds__(NW * 64, (NB == 1 ? 2 : 1)) void attn_bwd_dkdv_kern
     const float *lse2 = a.delta + (int64_t)a.B * a.H * a.Sq;   // written by the delta kernel
     const TileLaneOffsets lo = make_tile_offsets(lane);
     const uint32_t smem_base = lds_addr(&smem[0][0][0]), stat_base = lds_addr(&sstat[0][0][0]);
+    const uint32_t doc_base = lds_addr(&sdoc[0][0]);
+    constexpr bool has_docs = DOCS;
+    int jkey[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) jkey[nb] = wj0 + 32 * nb + l32;
 
     // Iteration `it` -> (query tile, query head).  Query tiles run from the LAST one
     // down and heads are the inner index, so every workgroup of this KV head that is
@@ -338,8 +269,13 @@ __global__ __launch_bounds__(NW * 64, (NB == 1 ? 2 : 1)) void attn_bwd_dkdv_kern
             const float *src = ((w >> 1) ? a.delta : lse2) + ((int64_t)b * a.H + hq) * a.Sq + i;
             __builtin_amdgcn_global_load_lds((glb_void_t *)src, (lds_void_t *)(&sstat[stage][w >> 1][32 * (w & 1)]), 4, 0, 0);
         }
+        if (DOCS && lane < 16) {          // wavefront w copies the document starts of 16 rows
+            const int i = min(i0 + 16 * w + lane, a.Sq - 1);
+            const int32_t *src = a.doc_start + (int64_t)b * a.Sq + i;
+            __builtin_amdgcn_global_load_lds((glb_void_t *)src, (lds_void_t *)(&sdoc[DOCS ? stage : 0][16 * w]), 4, 0, 0);
+        }
     };
-    constexpr int kLoadsPerIt = 5;     // vector-memory instructions one wavefront issues per iteration
+    // vector-memory instructions one wavefront issues per iteration: 5, or 6 with document starts
 
     // One iteration on a compile-time LDS stage, so that every fragment address is
     // (lane offset register) + (immediate).
@@ -347,22 +283,31 @@ __global__ __launch_bounds__(NW * 64, (NB == 1 ? 2 : 1)) void attn_bwd_dkdv_kern
         constexpr int STAGE = decltype(stage_tag)::value;
         // the copies for this iteration were issued two iterations ago; those of the next
         // one may stay in flight
-        if (it + 1 < n_it) wait_vmcnt<kLoadsPerIt>(); else wait_vmcnt<0>();
+        if (it + 1 >= n_it) wait_vmcnt<0>(); else if (has_docs) wait_vmcnt<6>(); else wait_vmcnt<5>();
         __syncthreads();
         if (it + 2 < n_it) issue(it + 2);
 
         const uint32_t qsm = smem_base + STAGE * (2 * kStageTileBytes), gsm = qsm + kStageTileBytes;
         const uint32_t stat_lane = stat_base + STAGE * (2 * kTile * 4) + half * 16;
+        const uint32_t ds_lane = doc_base + STAGE * (kTile * 4) + half * 16;
         const int i0 = (qt_hi - 1 - it / a.r) * kTile;
         const int pos0 = a.q_offset + i0;                                    // first query position of the tile
         const int pos1 = min(a.q_offset + min(a.Sq, i0 + kTile) - 1, q_len - 1);   // last live one
         const int wj1 = min(wj0 + WK, kv_len) - 1;                           // wavefront's last live key
-        const bool skip = wj1 < wj0 || pos1 < wj0 || pos0 > wj1 + weff - 1 || pos1 < pos0;
+        bool skip = wj1 < wj0 || pos1 < wj0 || pos0 > wj1 + weff - 1 || pos1 < pos0;
+        bool interior = (wj0 + WK - 1 <= pos0) && (wj0 > pos1 - weff) && (wj0 + WK <= kv_len) &&
+                        (a.q_offset + i0 + kTile - 1 <= pos1);
+        if constexpr (DOCS) {
+            // document starts never decrease along a row: the tile's first row has the smallest,
+            // its last row the largest (rows past the end repeat the last valid one)
+            const int ds_first = __builtin_amdgcn_readfirstlane(sdoc[STAGE][0]);
+            const int ds_last = __builtin_amdgcn_readfirstlane(sdoc[STAGE][kTile - 1]);
+            skip = skip || ds_first > wj1;
+            interior = interior && ds_last <= wj0;
+        }
         if (skip) return;
-        const bool interior = (wj0 + WK - 1 <= pos0) && (wj0 > pos1 - weff) && (wj0 + WK <= kv_len) &&
-                              (a.q_offset + i0 + kTile - 1 <= pos1);
         if (interior) {
-            dkdv_tile<false, NB>(qsm, gsm, stat_lane, lo, kf, vf, dk, dv, c, half, dead, 0u, 0, 0);
+            dkdv_tile<false, false, NB>(qsm, gsm, stat_lane, lo, kf, vf, dk, dv, c, half, dead, 0u, 0, 0, 0u, jkey);
         } else {
             int dbase[NB];
 #pragma unroll
@@ -371,7 +316,8 @@ __global__ __launch_bounds__(NW * 64, (NB == 1 ? 2 : 1)) void attn_bwd_dkdv_kern
                 dbase[nb] = (j < kv_len) ? pos0 - j : -0x40000000;
             }
             const int row_lim = (int)min((int64_t)kTile, min((int64_t)a.Sq, (int64_t)q_len - a.q_offset) - i0);
-            dkdv_tile<true, NB>(qsm, gsm, stat_lane, lo, kf, vf, dk, dv, c, half, dbase, (unsigned)weff, row_lim, wj0 - pos0);
+            dkdv_tile<true, DOCS, NB>(qsm, gsm, stat_lane, lo, kf, vf, dk, dv, c, half, dbase, (unsigned)weff, row_lim,
+                                      wj0 - pos0, ds_lane, jkey);
         }
     };
 
@@ -407,7 +353,7 @@ template <bool MASKED, int NQB>
 __device__ __forceinline__ void dq_tile(uint32_t ksm, uint32_t vsm, const TileLaneOffsets &lo, const bf16x8 (&qf)[NQB][4],
                                         const bf16x8 (&gf)[NQB][4], f32x16 (&dq)[NQB][2], const float (&lse2)[NQB],
                                         const float (&dlt)[NQB], float c, int lane, const int (&dbase)[NQB],
-                                        unsigned weff, int key_lim, int wrel) {
+                                        const unsigned (&wl)[NQB], unsigned weff, int key_lim, int wrel) {
     // wrel (masked variant only): (first query position of the wavefront) - (first key of the
     // tile); a 32-key half of the tile that no row of the wavefront can see is skipped.
     const int half = lane >> 5;
@@ -436,7 +382,7 @@ __device__ __forceinline__ void dq_tile(uint32_t ksm, uint32_t vsm, const TileLa
                 float pe = fast_exp2(fmaf(s[qb][i], c, -lse2[qb]));
                 if (MASKED) {
                     const int r = 32 * kb + crow(i, half);
-                    const bool vis = ((unsigned)(dbase[qb] - r) < weff) & (r < key_lim);
+                    const bool vis = ((unsigned)(dbase[qb] - r) < wl[qb]) & (r < key_lim);
                     pe = vis ? pe : 0.0f;
                 }
                 dp[qb][i] = pe * (dp[qb][i] + dlt[qb]);        // dlt holds -delta
@@ -488,7 +434,11 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_bwd_dq_kernel(co
     const int bpos1 = min(a.q_offset + min(a.Sq, (qt + 1) * BM) - 1, q_len - 1);
     const int hi = bpos1 >= bpos0 ? min(kv_len, bpos1 + 1) : 0;
     const int key_lo = max(0, bpos0 - weff + 1);
-    const int t_lo = key_lo / kTile;
+    const int32_t *dsrow = a.doc_start ? a.doc_start + (int64_t)b * a.Sq : nullptr;
+    const int ds_b0 = dsrow ? dsrow[min(qt * BM, a.Sq - 1)] : 0;
+    const int ds_w0 = dsrow ? dsrow[min(qw0, a.Sq - 1)] : 0;
+    const int ds_w1 = dsrow ? dsrow[min(qw0 + WM - 1, a.Sq - 1)] : 0;
+    const int t_lo = max(key_lo, ds_b0) / kTile;
     const int t_hi = hi > 0 ? (hi + kTile - 1) / kTile : 0;
 
     const int wpos0 = a.q_offset + qw0;
@@ -500,6 +450,7 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_bwd_dq_kernel(co
     bf16x8 qf[NQB][4], gf[NQB][4];
     float lse2[NQB], dlt[NQB];
     int pq[NQB];
+    unsigned wl[NQB];
 #pragma unroll
     for (int qb = 0; qb < NQB; ++qb) {
         const int row = qw0 + 32 * qb + l32;
@@ -525,6 +476,8 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_bwd_dq_kernel(co
         }
         const int p = a.q_offset + row;
         pq[qb] = (row_ok && p < q_len) ? p : -0x40000000;
+        wl[qb] = (unsigned)weff;
+        if (dsrow && row_ok) wl[qb] = (unsigned)min(weff, p - dsrow[row] + 1);
     }
 
     const float c = a.scale_log2;
@@ -551,17 +504,18 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_bwd_dq_kernel(co
         if (it + 2 < n_it) issue(it + 2);
         const uint32_t ksm = smem_base + STAGE * (2 * kStageTileBytes), vsm = ksm + kStageTileBytes;
         const int n0 = (t_lo + it) * kTile;
-        const bool skip = !active || n0 > wpos1 || (n0 + kTile - 1) < (wpos0 - weff + 1) || wpos1 < wpos0;
+        const bool skip = !active || n0 > wpos1 || (n0 + kTile - 1) < (wpos0 - weff + 1) || wpos1 < wpos0 ||
+                          (n0 + kTile - 1) < ds_w0;
         if (skip) return;
         const bool interior = (n0 + kTile - 1 <= wpos0) && (n0 > wpos1 - weff) && (n0 + kTile <= kv_len) &&
-                              (a.q_offset + qw0 + WM - 1 <= wpos1);
+                              (a.q_offset + qw0 + WM - 1 <= wpos1) && (n0 >= ds_w1);
         if (interior) {
-            dq_tile<false, NQB>(ksm, vsm, lo, qf, gf, dq, lse2, dlt, c, lane, pq, 0u, 0, 0);
+            dq_tile<false, NQB>(ksm, vsm, lo, qf, gf, dq, lse2, dlt, c, lane, pq, wl, 0u, 0, 0);
         } else {
             int dbase[NQB];
 #pragma unroll
             for (int qb = 0; qb < NQB; ++qb) dbase[qb] = pq[qb] - n0;
-            dq_tile<true, NQB>(ksm, vsm, lo, qf, gf, dq, lse2, dlt, c, lane, dbase, (unsigned)weff, kv_len - n0, wpos0 - n0);
+            dq_tile<true, NQB>(ksm, vsm, lo, qf, gf, dq, lse2, dlt, c, lane, dbase, wl, (unsigned)weff, kv_len - n0, wpos0 - n0);
         }
     };
 

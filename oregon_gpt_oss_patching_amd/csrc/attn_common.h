@@ -38,6 +38,7 @@ struct KArgs {
     const bf16 *q, *k, *v;
     const float *sinks;
     const int32_t *seqlens;
+    const int32_t *doc_start;   // optional (B, Sq): first key of each query's document
     bf16 *o;
     float *lse;
     const bf16 *d_o;

@@ -29,7 +29,9 @@ namespace gptoss {
 template <bool MASKED, int NQB>
 __device__ __forceinline__ void fwd_tile(uint32_t ksm, uint32_t vsm, const TileLaneOffsets &lo, const bf16x8 (&qf)[NQB][4],
                                          f32x16 (&o)[NQB][2], float (&m)[NQB], float (&l)[NQB], float c, int lane,
-                                         const int (&dbase)[NQB], unsigned weff, int key_lim, int wrel) {
+                                         const int (&dbase)[NQB], const unsigned (&wl)[NQB], unsigned weff, int key_lim,
+                                         int wrel) {
+    // wl[qb]: this lane's own window, min(window, distance back to the start of its document).
     // wrel (masked variant only): (first query position of the wavefront) - (first key of the
     // tile).  A 32-key half of the tile whose keys all lie in the future of every row of the
     // wavefront, or all fell out of every row's window, is skipped outright (no MFMA, no exp).
@@ -63,7 +65,7 @@ __device__ __forceinline__ void fwd_tile(uint32_t ksm, uint32_t vsm, const TileL
 #pragma unroll
                     for (int i = 0; i < 16; ++i) {
                         const int r = 32 * kb + crow(i, half);
-                        const bool vis = ((unsigned)(dbase[qb] - r) < weff) & (r < key_lim);
+                        const bool vis = ((unsigned)(dbase[qb] - r) < wl[qb]) & (r < key_lim);
                         s[kb][qb][i] = vis ? s[kb][qb][i] : -INFINITY;
                     }
                 }
@@ -150,7 +152,13 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_fwd_kernel(const
     const int bpos1 = min(a.q_offset + min(a.Sq, (qt + 1) * BM) - 1, q_len - 1);
     const int hi = bpos1 >= bpos0 ? min(kv_len, bpos1 + 1) : 0;   // no key at all for a fully padded tile
     const int key_lo = max(0, bpos0 - weff + 1);
-    const int t_lo = key_lo / kTile;
+    // packed rows: first key of the document of the workgroup's first row (document starts never
+    // decrease along a row), and of this wavefront's first and last rows
+    const int32_t *dsrow = a.doc_start ? a.doc_start + (int64_t)b * a.Sq : nullptr;
+    const int ds_b0 = dsrow ? dsrow[min(qt * BM, a.Sq - 1)] : 0;
+    const int ds_w0 = dsrow ? dsrow[min(qw0, a.Sq - 1)] : 0;
+    const int ds_w1 = dsrow ? dsrow[min(qw0 + WM - 1, a.Sq - 1)] : 0;
+    const int t_lo = max(key_lo, ds_b0) / kTile;
     const int t_hi = hi > 0 ? (hi + kTile - 1) / kTile : 0;
 
     // this wavefront's own row range (absolute positions)
@@ -163,6 +171,7 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_fwd_kernel(const
     // Q^T fragments (B operand), resident for the whole key loop
     bf16x8 qf[NQB][4];
     int pq[NQB];            // lane's query position per block, hugely negative when the row is dead
+    unsigned wl[NQB];       // lane's own window: min(window, distance back to its document's first key)
 #pragma unroll
     for (int qb = 0; qb < NQB; ++qb) {
         const int row = qw0 + 32 * qb + l32;
@@ -175,6 +184,8 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_fwd_kernel(const
         }
         const int p = a.q_offset + row;
         pq[qb] = (row < a.Sq && p < q_len) ? p : -0x40000000;
+        wl[qb] = (unsigned)weff;
+        if (dsrow && row < a.Sq) wl[qb] = (unsigned)min(weff, p - dsrow[row] + 1);
     }
 
     const float c = a.scale_log2;
@@ -208,17 +219,18 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_fwd_kernel(const
         const uint32_t ksm = smem_base + STAGE * (2 * kStageTileBytes), vsm = ksm + kStageTileBytes;
         const int n0 = (t_lo + it) * kTile;
         // tile classification for this wavefront: skip / interior / needs mask
-        const bool skip = !active || n0 > wpos1 || (n0 + kTile - 1) < (wpos0 - weff + 1) || wpos1 < wpos0;
+        const bool skip = !active || n0 > wpos1 || (n0 + kTile - 1) < (wpos0 - weff + 1) || wpos1 < wpos0 ||
+                          (n0 + kTile - 1) < ds_w0;
         if (skip) return;
         const bool interior = (n0 + kTile - 1 <= wpos0) && (n0 > wpos1 - weff) && (n0 + kTile <= kv_len) &&
-                              (a.q_offset + qw0 + WM - 1 <= wpos1);
+                              (a.q_offset + qw0 + WM - 1 <= wpos1) && (n0 >= ds_w1);
         if (interior) {
-            fwd_tile<false, NQB>(ksm, vsm, lo, qf, o, m, l, c, lane, pq, 0u, 0, 0);
+            fwd_tile<false, NQB>(ksm, vsm, lo, qf, o, m, l, c, lane, pq, wl, 0u, 0, 0);
         } else {
             int dbase[NQB];
 #pragma unroll
             for (int qb = 0; qb < NQB; ++qb) dbase[qb] = pq[qb] - n0;   // stays hugely negative for dead rows
-            fwd_tile<true, NQB>(ksm, vsm, lo, qf, o, m, l, c, lane, dbase, (unsigned)weff, kv_len - n0, wpos0 - n0);
+            fwd_tile<true, NQB>(ksm, vsm, lo, qf, o, m, l, c, lane, dbase, wl, (unsigned)weff, kv_len - n0, wpos0 - n0);
         }
     };
 

@@ -33,6 +33,7 @@ KArgs make_args(const gptoss_attn_params *p) {
     a.v = static_cast<const bf16 *>(p->v);
     a.sinks = p->sinks;
     a.seqlens = p->seqlens;
+    a.doc_start = p->doc_start;
     a.o = static_cast<bf16 *>(p->o);
     a.lse = p->lse;
     a.d_o = static_cast<const bf16 *>(p->d_o);
@@ -81,7 +82,7 @@ const char *gptoss_attn_status_string(int status) {
         case GPTOSS_ATTN_ERR_NULL_TENSOR: return "a required tensor pointer is NULL";
         case GPTOSS_ATTN_ERR_HEAD_DIM: return "head_dim must be 64";
         case GPTOSS_ATTN_ERR_HEADS: return "H and G must be positive and H divisible by G";
-        case GPTOSS_ATTN_ERR_SHAPE: return "B, Sq, Skv must be positive; window, q_offset non-negative; scale positive and finite";
+        case GPTOSS_ATTN_ERR_SHAPE: return "B, Sq, Skv must be positive; window, q_offset non-negative; scale positive and finite; doc_start needs Sq == Skv and q_offset == 0";
         case GPTOSS_ATTN_ERR_DTYPE: return "unsupported dtype";
         case GPTOSS_ATTN_ERR_ALIGNMENT: return "tensor base or stride is not 16-byte aligned";
         case GPTOSS_ATTN_ERR_STRIDE: return "sequence stride smaller than head_dim";
@@ -98,6 +99,7 @@ int gptoss_attn_validate(const gptoss_attn_params *p, int need_bwd) {
     if (p->H <= 0 || p->G <= 0 || p->H % p->G) return GPTOSS_ATTN_ERR_HEADS;
     if (p->B <= 0 || p->Sq <= 0 || p->Skv <= 0 || p->window < 0 || p->q_offset < 0) return GPTOSS_ATTN_ERR_SHAPE;
     if (!(p->scale > 0.0f) || !(p->scale < 3.0e38f)) return GPTOSS_ATTN_ERR_SHAPE;
+    if (p->doc_start && (p->Sq != p->Skv || p->q_offset != 0)) return GPTOSS_ATTN_ERR_SHAPE;
     const int eb = 2;
     int rc;
     if ((rc = check_tensor(p->q, p->q_stride, eb, p->D))) return rc;
@@ -158,7 +160,8 @@ int gptoss_attn_bwd_dkdv(const gptoss_attn_params *p, void *stream) {
     constexpr int kWaves = 4;                       // wavefronts per workgroup
     const int bn = 32 * kDkdvNB * kWaves;           // keys per workgroup
     const unsigned grid = (unsigned)(a.G * a.B * ((a.Skv + bn - 1) / bn));
-    hipLaunchKernelGGL((attn_bwd_dkdv_kernel<kWaves, kDkdvNB>), dim3(grid), dim3(64 * kWaves), 0, st, a);
+    if (a.doc_start) hipLaunchKernelGGL((attn_bwd_dkdv_kernel<kWaves, kDkdvNB, true>), dim3(grid), dim3(64 * kWaves), 0, st, a);
+    else hipLaunchKernelGGL((attn_bwd_dkdv_kernel<kWaves, kDkdvNB, false>), dim3(grid), dim3(64 * kWaves), 0, st, a);
     return launch_status();
 }
 

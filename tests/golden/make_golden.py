@@ -10,7 +10,8 @@ Run once, in the authoring container (needs `transformers`; nothing is fetched):
 The fixtures hold inputs' seed recipe and the expected outputs only.  The mask is
 built by transformers' own `eager_mask` from its own mask functions, i.e. the
 same additive finfo.min mask the model would hand to eager attention, including
-the 2-D padding mask for the padded-batch case.
+the 2-D padding mask for the padded-batch cases and the same-document mask that
+transformers derives from restarting position ids for the packed cases.
 """
 import os
 import sys
@@ -24,23 +25,33 @@ sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
 
 from oracle.eager_ref import make_inputs  # noqa: E402  (seed recipe only)
 
+# packed rows: document lengths per batch row (position ids restart at each document)
+PACKED = {"tiny_packed_full": [[20, 30, 14]], "tiny_packed_win8": [[5, 41, 18]]}
+
 CASES = [
     # name, seed, B, H, G, S, D, window, seqlens
     ("tiny_full", 11, 1, 8, 2, 64, 64, None, None),
     ("tiny_win8", 12, 1, 8, 2, 64, 64, 8, None),
     ("tiny_pad_full", 13, 2, 8, 2, 48, 64, None, [48, 29]),
     ("tiny_pad_win8", 14, 2, 8, 2, 48, 64, 8, [17, 48]),
+    ("tiny_packed_full", 15, 1, 8, 2, 64, 64, None, None),
+    ("tiny_packed_win8", 16, 1, 8, 2, 64, 64, 8, None),
     ("cfg1_full", 1, 1, 8, 2, 256, 64, None, None),
     ("cfg1_win32", 1, 1, 8, 2, 256, 64, 32, None),
 ]
 
 
-def run_case(seed, b, h, g, s, d, window, seqlens):
+def run_case(seed, b, h, g, s, d, window, seqlens, doc_lens=None):
     from transformers import masking_utils as mu
     from transformers.models.gpt_oss import modeling_gpt_oss as mg
 
     q, k, v, sinks, d_out = make_inputs(seed, b, h, g, s, d, torch.float32)
     fn = mu.causal_mask_function if window is None else mu.sliding_window_causal_mask_function(window)
+    if doc_lens is not None:
+        # transformers' own packed-sequence detection from position ids (masking_utils.py:728-757)
+        pos = torch.tensor([[p for n in lens for p in range(n)] for lens in doc_lens])
+        packed = mu.find_packed_sequence_indices(pos)
+        fn = mu.and_masks(fn, mu.packed_sequence_mask_function(packed))
     pad2d = None
     if seqlens is not None:
         pad2d = torch.arange(s).view(1, s) < torch.tensor(seqlens).view(b, 1)
@@ -61,9 +72,10 @@ def run_case(seed, b, h, g, s, d, window, seqlens):
 
 def main():
     for name, seed, b, h, g, s, d, window, seqlens in CASES:
-        out, dq, dk, dv, ds = run_case(seed, b, h, g, s, d, window, seqlens)
+        out, dq, dk, dv, ds = run_case(seed, b, h, g, s, d, window, seqlens, PACKED.get(name))
         meta = dict(seed=seed, B=b, H=h, G=g, S=s, D=d, window=window or 0,
-                    seqlens=np.array(seqlens if seqlens else [], dtype=np.int32))
+                    seqlens=np.array(seqlens if seqlens else [], dtype=np.int32),
+                    doc_lens=np.array(PACKED.get(name, []), dtype=np.int32))
         if s > 64:
             # config-1 size: keep norms and a fixed strided sample, not full tensors
             def samp(t):

@@ -47,7 +47,7 @@ def test_struct_mirror_matches_header_field_order():
         for part in decl.split(","):
             names.append(re.findall(r"[A-Za-z_][A-Za-z_0-9]*", part)[-1])
     assert names == [f[0] for f in _lib.Params._fields_]
-    assert ctypes.sizeof(_lib.Params) == 344
+    assert ctypes.sizeof(_lib.Params) == 352
 
 
 def _valid_params():
@@ -91,6 +91,8 @@ def test_validate_accepts_good_params():
     (lambda p: setattr(p, "k", 0x1008), -7),
     (lambda p: setattr(p.v_stride, "s", 68), -7),
     (lambda p: setattr(p.v_stride, "s", 32), -8),
+    (lambda p: (setattr(p, "doc_start", 0x2000), setattr(p, "q_offset", 4)), -5),
+    (lambda p: (setattr(p, "doc_start", 0x2000), setattr(p, "Skv", 256)), -5),
 ])
 def test_validate_error_codes(mutate, code):
     p = _valid_params()

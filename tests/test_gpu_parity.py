@@ -48,25 +48,26 @@ def check(name, got, ref, rel=1e-2, atol=2e-2):
         assert bool((err <= bound).all()), (name, "max-abs", float(err.max()), float(ref.abs().max()))
 
 
-def run_hip(A, q, k, v, sinks, d_out, window, q_offset=0, seqlens=None):
+def run_hip(A, q, k, v, sinks, d_out, window, q_offset=0, seqlens=None, doc_start=None):
     qd, kd, vd, sd, dod = (t.to(DEV) for t in (q, k, v, sinks, d_out))
-    o, lse = A.attention_forward(qd, kd, vd, sd, SCALE, window, q_offset, seqlens)
-    dq, dk, dv, ds = A.attention_backward(qd, kd, vd, sd, o, lse, dod, SCALE, window, q_offset, seqlens)
+    o, lse = A.attention_forward(qd, kd, vd, sd, SCALE, window, q_offset, seqlens, doc_start)
+    dq, dk, dv, ds = A.attention_backward(qd, kd, vd, sd, o, lse, dod, SCALE, window, q_offset, seqlens,
+                                          doc_start=doc_start)
     torch.cuda.synchronize()
     return o, lse, dq, dk, dv, ds
 
 
-def oracle_eager(q, k, v, sinks, d_out, window, q_offset=0, seqlens=None):
+def oracle_eager(q, k, v, sinks, d_out, window, q_offset=0, seqlens=None, doc_start=None):
     f = [t.float() for t in (q, k, v, sinks, d_out)]
-    out, dq, dk, dv, ds = E.eager_attention_grads(*f, SCALE, window, q_offset, seqlens)
-    lse = E.logsumexp_rows(f[0], f[1], f[3], SCALE, window, q_offset, seqlens)
+    out, dq, dk, dv, ds = E.eager_attention_grads(*f, SCALE, window, q_offset, seqlens, doc_start)
+    lse = E.logsumexp_rows(f[0], f[1], f[3], SCALE, window, q_offset, seqlens, doc_start)
     return out, lse, dq, dk, dv, ds
 
 
-def oracle_tiled(q, k, v, sinks, d_out, window, q_offset=0, seqlens=None):
+def oracle_tiled(q, k, v, sinks, d_out, window, q_offset=0, seqlens=None, doc_start=None):
     f = [t.float() for t in (q, k, v, sinks, d_out)]
-    o, lse = T.tiled_fwd(f[0], f[1], f[2], f[3], SCALE, window, q_offset, seqlens)
-    dq, dk, dv, ds, _ = T.tiled_bwd(f[0], f[1], f[2], f[3], o, lse, f[4], SCALE, window, q_offset, seqlens)
+    o, lse = T.tiled_fwd(f[0], f[1], f[2], f[3], SCALE, window, q_offset, seqlens, doc_start)
+    dq, dk, dv, ds, _ = T.tiled_bwd(f[0], f[1], f[2], f[3], o, lse, f[4], SCALE, window, q_offset, seqlens, doc_start)
     return o, lse, dq, dk, dv, ds
 
 
@@ -257,3 +258,55 @@ def test_window_ge_seq_equals_full(A):
     for w in (200, 4096):
         for x, y in zip(a, run_hip(A, *inp, w)):
             assert torch.equal(x, y)
+
+
+PACKED = [
+    # S, window, document lengths per row
+    (64, None, [[20, 30, 14]]),
+    (200, None, [[70, 3, 127], [200]]),
+    (333, 32, [[1, 100, 64, 168]]),
+    (512, 128, [[130, 126, 256], [64, 64, 384]]),
+    (300, None, [[299, 1]]),
+]
+
+
+@pytest.mark.parametrize("s,w,lens", PACKED)
+def test_packed_rows_vs_eager_oracle(A, s, w, lens):
+    """Rows packed from several documents: with doc_start the documents do not see each other."""
+    b = len(lens)
+    inp = E.make_inputs(200 + s, b, 16, 2, s, 64, torch.bfloat16)
+    ds = E.doc_start_from_lengths(lens, s)
+    compare_all(run_hip(A, *inp, w, 0, None, ds.to(DEV)), oracle_eager(*inp, w, 0, None, ds))
+
+
+def test_packed_rows_s4096_vs_tiled_oracle(A):
+    """GPT-OSS-20B head shape, S=4096 packed from ragged documents, both layer types, one KV group."""
+    s = 4096
+    gen = torch.Generator().manual_seed(9)
+    cuts = sorted(set(torch.randint(1, s, (9,), generator=gen).tolist()))
+    lens = [b_ - a_ for a_, b_ in zip([0] + cuts, cuts + [s])]
+    ds = E.doc_start_from_lengths([lens], s)
+    q, k, v, sinks, d_out = E.make_inputs(9, 1, 64, 8, s, 64, torch.bfloat16)
+    for w in (128, None):
+        o, lse, dq, dk, dv, dsk = run_hip(A, q, k, v, sinks, d_out, w, 0, None, ds.to(DEV))
+        g = 3
+        hs = slice(8 * g, 8 * g + 8)
+        ref = oracle_tiled(q[:, hs], k[:, g:g + 1], v[:, g:g + 1], sinks[hs], d_out[:, :, hs], w, 0, None, ds)
+        compare_all((o[:, :, hs], lse[:, hs], dq[:, hs], dk[:, g:g + 1], dv[:, g:g + 1], dsk[hs]), ref)
+
+
+def test_doc_start_from_position_ids(A):
+    pos = torch.tensor([[0, 1, 2, 0, 1, 0, 1, 2, 3], [0, 1, 2, 3, 4, 5, 6, 7, 8]], device=DEV)
+    ds = A.doc_start_from_position_ids(pos)
+    assert ds.tolist() == [[0, 0, 0, 3, 3, 5, 5, 5, 5], [0] * 9] and ds.dtype == torch.int32
+
+
+def test_transformers_packed_golden(A, golden_dir):
+    for name in ("tiny_packed_full", "tiny_packed_win8"):
+        z = np.load(os.path.join(golden_dir, f"{name}.npz"))
+        w = int(z["window"]) or None
+        ds = E.doc_start_from_lengths(z["doc_lens"].tolist(), 64).to(DEV)
+        inp = E.make_inputs(int(z["seed"]), 1, 8, 2, 64, 64, torch.float32)
+        o, lse, dq, dk, dv, dsk = run_hip(A, *(t.to(torch.bfloat16) for t in inp), w, 0, None, ds)
+        for n, t_ in (("out", o), ("dq", dq), ("dk", dk), ("dv", dv)):
+            assert rel_l2(t_.float().cpu(), torch.from_numpy(z[n])) < 1.5e-2, (name, n)

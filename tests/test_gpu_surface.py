@@ -186,3 +186,59 @@ def test_mask_free_padding_path_matches_masked_model():
         finally:
             patching.unpatch_flash_attention()
     assert abs(loss_p - loss_e) < 2e-2 * abs(loss_e), (loss_e, loss_p)
+
+
+def test_float32_tensors_are_accepted_at_bf16_accuracy():
+    """Config 1 as given (fp32 tensors): accepted, computed in bf16, results returned in fp32."""
+    import oregon_gpt_oss_patching_amd as A
+    q, k, v, sinks, d_out = E.make_inputs(1, 1, 8, 2, 256, 64, torch.float32)
+    for w in (None, 32):
+        ref = E.eager_attention_grads(q, k, v, sinks, d_out, SCALE, w)
+        qd, kd, vd, sd = (t.to(DEV).requires_grad_(True) for t in (q, k, v, sinks))
+        out = A.attention(qd, kd, vd, sd, SCALE, w, None)
+        assert out.dtype == torch.float32
+        out.backward(d_out.to(DEV))
+        for g, r in zip((out, qd.grad, kd.grad, vd.grad, sd.grad), ref):
+            assert g.dtype == torch.float32
+            assert rel_l2(g.detach().cpu(), r) < 1e-2
+
+
+def test_packed_rows_through_the_patched_model():
+    """Packed rows (position ids restarting inside a row).  The stock GPT-OSS eager path of this
+    transformers version does not pass position ids to its mask builder, so, like the reference,
+    it lets documents see each other; the default patch must match it.  With
+    respect_packing=True the patched model must instead match the eager model given
+    transformers' own same-document masks."""
+    from transformers import masking_utils as mu
+    from oregon_gpt_oss_patching_amd import patching
+    sft_bench, model, params = _tiny_lora_model()
+    s = 192
+    ids = torch.randint(0, 512, (1, s), device=DEV)
+    lens = [50, 100, 42]
+    pos = torch.tensor([[p for n in lens for p in range(n)]], device=DEV)
+    packed = mu.find_packed_sequence_indices(pos.cpu())
+    doc = mu.packed_sequence_mask_function(packed)
+    masks = {
+        "full_attention": mu.eager_mask(1, s, s, mask_function=mu.and_masks(mu.causal_mask_function, doc),
+                                        dtype=torch.bfloat16).to(DEV),
+        "sliding_attention": mu.eager_mask(1, s, s, mask_function=mu.and_masks(
+            mu.sliding_window_causal_mask_function(model.config.sliding_window), doc), dtype=torch.bfloat16).to(DEV),
+    }
+    free = sft_bench.mask_free_attention_mask(None)
+    model.eval()
+    with torch.no_grad():
+        ref_leaky = model(input_ids=ids, position_ids=pos).logits.float().cpu()
+        ref_docs = model(input_ids=ids, position_ids=pos, attention_mask=masks).logits.float().cpu()
+        patching.patch_flash_attention(respect_packing=True)
+        try:
+            got_docs = model(input_ids=ids, position_ids=pos, attention_mask=free).logits.float().cpu()
+        finally:
+            patching.unpatch_flash_attention()
+        patching.patch_flash_attention()
+        try:
+            got_leaky = model(input_ids=ids, position_ids=pos, attention_mask=free).logits.float().cpu()
+        finally:
+            patching.unpatch_flash_attention()
+    assert rel_l2(ref_docs[:, 60:], ref_leaky[:, 60:]) > 0.1          # the two semantics really differ
+    assert rel_l2(got_leaky, ref_leaky) < 3e-2
+    assert rel_l2(got_docs, ref_docs) < 3e-2

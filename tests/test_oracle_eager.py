@@ -167,3 +167,33 @@ def test_pair_count_and_flops():
     assert E.allowed_mask(256, 256, 32).sum().item() == 7696
     f = E.attention_flops(1, 64, 64, E.pair_count(16384, None))
     assert abs(f["total"] - 7.697e12) / 7.697e12 < 1e-3
+
+
+@pytest.mark.parametrize("name", ["tiny_packed_full", "tiny_packed_win8"])
+def test_golden_packed_sequences(golden_dir, name):
+    """Packed rows: transformers builds the same-document mask from position ids; the oracle
+    takes the equivalent document-start index per token."""
+    z, seed, b, h, g, s, d, w, sl = _load(golden_dir, name)
+    ds = E.doc_start_from_lengths(z["doc_lens"].tolist(), s)
+    q, k, v, sinks, d_out = E.make_inputs(seed, b, h, g, s, d)
+    got = E.eager_attention_grads(q, k, v, sinks, d_out, SCALE, w, 0, None, ds)
+    for name_, mine, gold in zip(("out", "dq", "dk", "dv", "dsinks"), got, (z["out"], z["dq"], z["dk"], z["dv"], z["dsinks"])):
+        gold = torch.as_tensor(gold)
+        assert torch.allclose(mine, gold, rtol=1e-4, atol=2e-5), (name_, float((mine - gold).abs().max()))
+    # and it differs from the unpacked result, so the fixture does exercise the document mask
+    plain = E.eager_attention(q, k, v, sinks, SCALE, w)
+    assert not torch.allclose(plain, got[0], atol=1e-3)
+
+
+def test_packed_row_equals_separate_documents():
+    """Each document of a packed row attends as if it were alone."""
+    lens = [7, 12, 5]
+    q, k, v, sinks, _ = E.make_inputs(13, 1, 4, 2, 24, 64, torch.float64)
+    ds = E.doc_start_from_lengths([lens], 24)
+    for w in (None, 4):
+        packed = E.eager_attention(q, k, v, sinks, SCALE, w, doc_start=ds)
+        pos = 0
+        for n in lens:
+            alone = E.eager_attention(q[:, :, pos:pos + n], k[:, :, pos:pos + n], v[:, :, pos:pos + n], sinks, SCALE, w)
+            assert torch.allclose(packed[:, pos:pos + n], alone, atol=1e-12)
+            pos += n
