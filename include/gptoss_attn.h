@@ -54,8 +54,9 @@ extern "C" {
 #define GPTOSS_ATTN_ABI_VERSION 2
 
 enum gptoss_attn_dtype {
-    GPTOSS_ATTN_BF16 = 0, /* 2-byte bfloat16 tensors, fp32 accumulation */
-    GPTOSS_ATTN_FP32 = 1  /* 4-byte float tensors (the reference's fp32 mode) */
+    GPTOSS_ATTN_BF16 = 0, /* 2-byte bfloat16 tensors, bf16 MFMA products, fp32 accumulation: the fast path */
+    GPTOSS_ATTN_FP32 = 1  /* 4-byte float tensors, fp32 MFMA products (the reference's fp32 mode,
+                             attention_kernel.py is dtype-generic): built for exactness, not tuned */
 };
 
 enum gptoss_attn_status {
@@ -108,6 +109,14 @@ int gptoss_attn_version(void);
 
 /* Text for a status code returned by any entry point (never NULL). */
 const char *gptoss_attn_status_string(int status);
+
+/*
+ * Bytes of the `delta` scratch buffer the backward entry points need for these shapes
+ * (2 * B * H * Sq floats); 0 for a NULL or shapeless params.  The reference allocates its
+ * counterpart itself (`delta = torch.empty_like(M)`, attention_kernel.py:303); here the caller
+ * owns it.  Host-only.
+ */
+size_t gptoss_attn_workspace_bytes(const gptoss_attn_params *params);
 
 /*
  * Forward: O and logsumexp.  Replaces the `_attn_fwd` launch in

@@ -20,6 +20,7 @@ EXPORTS = (
     "gptoss_attn_version",
     "gptoss_attn_status_string",
     "gptoss_attn_validate",
+    "gptoss_attn_workspace_bytes",
     "gptoss_attn_fwd",
     "gptoss_attn_bwd_preprocess",
     "gptoss_attn_bwd_dkdv",
@@ -83,6 +84,8 @@ def load() -> ctypes.CDLL:
         lib.gptoss_attn_status_string.argtypes = [ctypes.c_int]
         lib.gptoss_attn_validate.restype = ctypes.c_int
         lib.gptoss_attn_validate.argtypes = [ctypes.POINTER(Params), ctypes.c_int]
+        lib.gptoss_attn_workspace_bytes.restype = ctypes.c_size_t
+        lib.gptoss_attn_workspace_bytes.argtypes = [ctypes.POINTER(Params)]
         for name in ("gptoss_attn_fwd", "gptoss_attn_bwd_preprocess", "gptoss_attn_bwd_dkdv",
                      "gptoss_attn_bwd_dq", "gptoss_attn_bwd"):
             fn = getattr(lib, name)

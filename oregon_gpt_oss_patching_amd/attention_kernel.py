@@ -21,16 +21,16 @@ an optional `seqlens` (right-padding lengths) is accepted.
 """
 from __future__ import annotations
 
-from typing import Optional
+from typing import Optional, Tuple
 
 import torch
 
 from . import _lib
 
 __all__ = ["attention", "triton_flash_attention", "hip_flash_attention", "attention_forward", "attention_backward",
-           "doc_start_from_position_ids"]
+           "doc_start_from_position_ids", "OP_NAMESPACE"]
 
-_DTYPES = {torch.bfloat16: _lib.DTYPE_BF16}
+_DTYPES = {torch.bfloat16: _lib.DTYPE_BF16, torch.float32: _lib.DTYPE_FP32}
 
 # When True the Hugging Face adapter masks across documents of packed rows (from the
 # `position_ids` it is handed).  False reproduces the reference, which ignores position ids.
@@ -56,11 +56,13 @@ def _set(st, triple):
     st.b, st.h, st.s = (int(x) for x in triple)
 
 
-def _check_inputs(q, k, v, sinks):
+def _check_inputs(q, k, v, sinks, allow_cast=False):
     if not (q.is_cuda and k.is_cuda and v.is_cuda):
         raise RuntimeError("gptoss attention runs on the GPU only (HIP kernels); got a CPU tensor")
-    if q.dtype not in _DTYPES or k.dtype != q.dtype or v.dtype != q.dtype:
-        raise RuntimeError(f"unsupported dtypes {q.dtype}/{k.dtype}/{v.dtype}: bfloat16 tensors are required")
+    ok_dtypes = tuple(_DTYPES) + ((torch.float16,) if allow_cast else ())
+    if q.dtype not in ok_dtypes or k.dtype != q.dtype or v.dtype != q.dtype:
+        raise RuntimeError(f"unsupported dtypes {q.dtype}/{k.dtype}/{v.dtype}: "
+                           "q, k, v must all be bfloat16 or all be float32")
     if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
         raise RuntimeError("q must be (B,H,S,D) and k, v (B,G,S_kv,D)")
     if k.shape != v.shape or q.shape[0] != k.shape[0] or q.shape[3] != k.shape[3]:
@@ -155,7 +157,10 @@ def attention_backward(q, k, v, sinks, o, lse, d_o, sm_scale, window=None, q_off
     dq = torch.empty((b, h, sq, d), dtype=q.dtype, device=q.device)
     dk = torch.empty(k.shape, dtype=k.dtype, device=q.device)
     dv = torch.empty(v.shape, dtype=v.dtype, device=q.device)
-    delta = torch.empty((2, b, h, sq), dtype=torch.float32, device=q.device)   # [delta; lse*log2e]
+    p0 = _lib.new_params()
+    p0.B, p0.H, p0.Sq = b, h, sq
+    delta = torch.empty((_lib.load().gptoss_attn_workspace_bytes(p0) // 4,), dtype=torch.float32,
+                        device=q.device)                                       # [-delta; lse*log2e]
     dsinks = torch.empty((h,), dtype=torch.float32, device=q.device) if need_dsinks else None
     with torch.cuda.device(q.device):
         p = _base_params(q, k, v, sinks32, sl, sm_scale, window, q_offset, ds)
@@ -173,42 +178,83 @@ def attention_backward(q, k, v, sinks, o, lse, d_o, sm_scale, window=None, q_off
     return dq, dk, dv, dsinks
 
 
+# ---- torch custom ops --------------------------------------------------------------------
+# The two library calls are registered as opaque PyTorch operators, `gptoss_attn::fwd` and
+# `gptoss_attn::bwd`, with shape-only ("fake") implementations, so that tracing tools
+# (torch.compile, FakeTensorMode, activation-checkpoint replay) see one node per call and never
+# look inside.  The autograd.Function below calls through them.
+OP_NAMESPACE = "gptoss_attn"
+
+
+@torch.library.custom_op(f"{OP_NAMESPACE}::fwd", mutates_args=(), device_types="cuda")
+def _op_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, sinks: Optional[torch.Tensor], sm_scale: float,
+            window: int, q_offset: int, seqlens: Optional[torch.Tensor],
+            doc_start: Optional[torch.Tensor]) -> Tuple[torch.Tensor, torch.Tensor]:
+    return attention_forward(q, k, v, sinks, sm_scale, window, q_offset, seqlens, doc_start)
+
+
+@_op_fwd.register_fake
+def _op_fwd_fake(q, k, v, sinks, sm_scale, window, q_offset, seqlens, doc_start):
+    b, h, sq, d = q.shape
+    return q.new_empty((b, sq, h, d)), q.new_empty((b, h, sq), dtype=torch.float32)
+
+
+@torch.library.custom_op(f"{OP_NAMESPACE}::bwd", mutates_args=(), device_types="cuda")
+def _op_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, sinks: Optional[torch.Tensor], o: torch.Tensor,
+            lse: torch.Tensor, d_o: torch.Tensor, sm_scale: float, window: int, q_offset: int,
+            seqlens: Optional[torch.Tensor], doc_start: Optional[torch.Tensor],
+            need_dsinks: bool) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+    dq, dk, dv, dsinks = attention_backward(q, k, v, sinks, o, lse, d_o, sm_scale, window, q_offset, seqlens,
+                                            need_dsinks=need_dsinks, doc_start=doc_start)
+    if dsinks is None:      # an operator cannot return None: an empty tensor stands for "not requested"
+        dsinks = torch.empty((0,), dtype=torch.float32, device=q.device)
+    return dq, dk, dv, dsinks
+
+
+@_op_bwd.register_fake
+def _op_bwd_fake(q, k, v, sinks, o, lse, d_o, sm_scale, window, q_offset, seqlens, doc_start, need_dsinks):
+    return (torch.empty_like(q, memory_format=torch.contiguous_format),
+            torch.empty_like(k, memory_format=torch.contiguous_format),
+            torch.empty_like(v, memory_format=torch.contiguous_format),
+            q.new_empty((q.shape[1] if need_dsinks else 0,), dtype=torch.float32))
+
+
 class _attention(torch.autograd.Function):
     """Same argument list and gradient tuple as the reference's `_attention`
     (attention_kernel.py:220-344), plus optional trailing `seqlens` and `doc_start`.
 
-    The kernels compute on bfloat16 tensors.  float32 / float16 tensors are accepted for
-    convenience (the reference runs them natively): they are rounded to bfloat16 on the
-    way in and the results cast back, so their accuracy is bfloat16's, not float32's."""
+    bfloat16 tensors take the tuned bf16-MFMA kernels and float32 tensors the float32 kernels
+    (exact to float32 rounding, not tuned for speed).  float16 tensors are accepted for
+    convenience: they are rounded to bfloat16 on the way in and the results cast back."""
 
     @staticmethod
     def forward(ctx, q, k, v, sinks, sm_scale, bandwidth, start_q, seqlens=None, doc_start=None):
+        _check_inputs(q, k, v, sinks, allow_cast=True)
         ctx.in_dtypes = (q.dtype, k.dtype, v.dtype)
-        if q.dtype in (torch.float32, torch.float16):
+        if q.dtype == torch.float16:
             q, k, v = (t.to(torch.bfloat16) for t in (q, k, v))
         q_offset = 0
         if start_q is not None:
             q_offset = int(start_q.item()) if torch.is_tensor(start_q) else int(start_q)
-        if doc_start is not None:
-            doc_start = _prep_doc_start(doc_start, q)
-        o, lse = attention_forward(q, k, v, sinks, sm_scale, bandwidth, q_offset, seqlens, doc_start)
-        ctx.save_for_backward(q, k, v, sinks, o, lse, seqlens if torch.is_tensor(seqlens) else None, doc_start)
-        ctx.seqlens_list = None if torch.is_tensor(seqlens) else seqlens
-        ctx.sm_scale = sm_scale
-        ctx.bandwidth = bandwidth
+        seqlens = _prep_seqlens(seqlens, q.device, q.shape[0])
+        doc_start = _prep_doc_start(doc_start, q)
+        window = int(bandwidth or 0)
+        sinks_in = None if sinks is None else sinks.detach()
+        o, lse = _op_fwd(q, k, v, sinks_in, float(sm_scale), window, q_offset, seqlens, doc_start)
+        ctx.save_for_backward(q, k, v, sinks, o, lse, seqlens, doc_start)
+        ctx.sm_scale = float(sm_scale)
+        ctx.window = window
         ctx.q_offset = q_offset
         return o.to(ctx.in_dtypes[0])
 
     @staticmethod
     def backward(ctx, do):
-        q, k, v, sinks, o, lse, seqlens_t, doc_start = ctx.saved_tensors
-        seqlens = seqlens_t if seqlens_t is not None else ctx.seqlens_list
+        q, k, v, sinks, o, lse, seqlens, doc_start = ctx.saved_tensors
         need_ds = sinks is not None and ctx.needs_input_grad[3]
-        dq, dk, dv, dsinks = attention_backward(
-            q, k, v, sinks, o, lse, do.to(q.dtype), ctx.sm_scale, ctx.bandwidth, ctx.q_offset, seqlens,
-            need_dsinks=need_ds, doc_start=doc_start)
-        if dsinks is not None:
-            dsinks = dsinks.to(sinks.dtype).view_as(sinks)
+        sinks_in = None if sinks is None else sinks.detach()
+        dq, dk, dv, dsinks = _op_bwd(q, k, v, sinks_in, o, lse, do.to(q.dtype), ctx.sm_scale, ctx.window,
+                                     ctx.q_offset, seqlens, doc_start, need_ds)
+        dsinks = dsinks.to(sinks.dtype).view_as(sinks) if need_ds else None
         qd, kd, vd = ctx.in_dtypes
         return dq.to(qd), dk.to(kd), dv.to(vd), dsinks, None, None, None, None, None
 

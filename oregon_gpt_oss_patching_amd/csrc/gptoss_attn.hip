@@ -6,6 +6,7 @@
 #include "../../include/gptoss_attn.h"
 #include "attn_bwd.h"
 #include "attn_common.h"
+#include "attn_f32.h"
 #include "attn_fwd.h"
 
 using namespace gptoss;
@@ -64,6 +65,9 @@ int query_blocks_for(int window) { return (window > 0 && window <= 1024) ? 1 : 2
 // 32-key blocks per wavefront in the dK/dV kernel
 constexpr int kDkdvNB = 1;
 
+// workgroups of four independent wavefronts for the float32 kernels
+unsigned f32_grid(int64_t waves) { return (unsigned)((waves + 3) / 4); }
+
 int launch_status() {
     const hipError_t e = hipGetLastError();
     return e == hipSuccess ? GPTOSS_ATTN_OK : static_cast<int>(e);
@@ -94,13 +98,13 @@ const char *gptoss_attn_status_string(int status) {
 int gptoss_attn_validate(const gptoss_attn_params *p, int need_bwd) {
     if (!p) return GPTOSS_ATTN_ERR_NULL_PARAMS;
     if (p->struct_size != sizeof(gptoss_attn_params)) return GPTOSS_ATTN_ERR_ABI;
-    if (p->dtype != GPTOSS_ATTN_BF16) return GPTOSS_ATTN_ERR_DTYPE;
+    if (p->dtype != GPTOSS_ATTN_BF16 && p->dtype != GPTOSS_ATTN_FP32) return GPTOSS_ATTN_ERR_DTYPE;
     if (p->D != kD) return GPTOSS_ATTN_ERR_HEAD_DIM;
     if (p->H <= 0 || p->G <= 0 || p->H % p->G) return GPTOSS_ATTN_ERR_HEADS;
     if (p->B <= 0 || p->Sq <= 0 || p->Skv <= 0 || p->window < 0 || p->q_offset < 0) return GPTOSS_ATTN_ERR_SHAPE;
     if (!(p->scale > 0.0f) || !(p->scale < 3.0e38f)) return GPTOSS_ATTN_ERR_SHAPE;
     if (p->doc_start && (p->Sq != p->Skv || p->q_offset != 0)) return GPTOSS_ATTN_ERR_SHAPE;
-    const int eb = 2;
+    const int eb = p->dtype == GPTOSS_ATTN_FP32 ? 4 : 2;
     int rc;
     if ((rc = check_tensor(p->q, p->q_stride, eb, p->D))) return rc;
     if ((rc = check_tensor(p->k, p->k_stride, eb, p->D))) return rc;
@@ -117,11 +121,20 @@ int gptoss_attn_validate(const gptoss_attn_params *p, int need_bwd) {
     return GPTOSS_ATTN_OK;
 }
 
+size_t gptoss_attn_workspace_bytes(const gptoss_attn_params *p) {
+    if (!p || p->B <= 0 || p->H <= 0 || p->Sq <= 0) return 0;
+    return (size_t)2 * sizeof(float) * (size_t)p->B * (size_t)p->H * (size_t)p->Sq;
+}
+
 int gptoss_attn_fwd(const gptoss_attn_params *p, void *stream) {
     const int rc = gptoss_attn_validate(p, 0);
     if (rc) return rc;
     const KArgs a = make_args(p);
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (p->dtype == GPTOSS_ATTN_FP32) {
+        hipLaunchKernelGGL(attn_f32_fwd_kernel, dim3(f32_grid((int64_t)a.B * a.H * ((a.Sq + 31) / 32))), dim3(256), 0, st, a);
+        return launch_status();
+    }
     const int hpb = hpb_for(a.r), qb = query_blocks_for(a.window);
     const int bm = 32 * qb * (4 / hpb);
     const int n_hc = (a.r + hpb - 1) / hpb;
@@ -142,7 +155,10 @@ int gptoss_attn_bwd_preprocess(const gptoss_attn_params *p, void *stream) {
     const KArgs a = make_args(p);
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int64_t rows = (int64_t)a.B * a.H * a.Sq;
-    hipLaunchKernelGGL(attn_bwd_delta_kernel, dim3((unsigned)((rows + 127) / 128)), dim3(256), 0, st, a);
+    if (p->dtype == GPTOSS_ATTN_FP32)
+        hipLaunchKernelGGL(attn_f32_delta_kernel, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st, a);
+    else
+        hipLaunchKernelGGL(attn_bwd_delta_kernel, dim3((unsigned)((rows + 127) / 128)), dim3(256), 0, st, a);
     int s = launch_status();
     if (s) return s;
     if (a.dsinks) {
@@ -157,6 +173,10 @@ int gptoss_attn_bwd_dkdv(const gptoss_attn_params *p, void *stream) {
     if (rc) return rc;
     const KArgs a = make_args(p);
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (p->dtype == GPTOSS_ATTN_FP32) {
+        hipLaunchKernelGGL(attn_f32_dkdv_kernel, dim3(f32_grid((int64_t)a.B * a.G * ((a.Skv + 31) / 32))), dim3(256), 0, st, a);
+        return launch_status();
+    }
     constexpr int kWaves = 4;                       // wavefronts per workgroup
     const int bn = 32 * kDkdvNB * kWaves;           // keys per workgroup
     const unsigned grid = (unsigned)(a.G * a.B * ((a.Skv + bn - 1) / bn));
@@ -170,6 +190,10 @@ int gptoss_attn_bwd_dq(const gptoss_attn_params *p, void *stream) {
     if (rc) return rc;
     const KArgs a = make_args(p);
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (p->dtype == GPTOSS_ATTN_FP32) {
+        hipLaunchKernelGGL(attn_f32_dq_kernel, dim3(f32_grid((int64_t)a.B * a.H * ((a.Sq + 31) / 32))), dim3(256), 0, st, a);
+        return launch_status();
+    }
     const int hpb = hpb_for(a.r), qb = query_blocks_for(a.window);
     const int bm = 32 * qb * (4 / hpb);
     const int n_hc = (a.r + hpb - 1) / hpb;

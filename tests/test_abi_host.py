@@ -132,3 +132,26 @@ def test_call_raises_with_status_text():
     with pytest.raises(_lib.GptossAttnError) as ei:
         _lib.call("gptoss_attn_fwd", p, 0)
     assert ei.value.status == -4 and "divisible" in str(ei.value)
+
+
+def test_validate_float32_params_and_their_alignment_rule():
+    """float32 tensors: rows must still start on 16-byte boundaries, i.e. strides are multiples
+    of 4 elements (8 for bf16): a stride of 68 floats is fine, 66 is not."""
+    p = _valid_params()
+    p.dtype = _lib.DTYPE_FP32
+    assert _validate(p) == 0
+    p.v_stride.s = 68
+    assert _validate(p) == 0
+    p.v_stride.s = 66
+    assert _validate(p) == -7
+
+
+def test_workspace_bytes():
+    lib = _lib.load()
+    p = _valid_params()
+    assert lib.gptoss_attn_workspace_bytes(ctypes.byref(p)) == 2 * 4 * 1 * 8 * 128
+    p.B, p.H, p.Sq = 4, 64, 16384
+    assert lib.gptoss_attn_workspace_bytes(ctypes.byref(p)) == 2 * 4 * 4 * 64 * 16384
+    p.Sq = 0
+    assert lib.gptoss_attn_workspace_bytes(ctypes.byref(p)) == 0
+    assert lib.gptoss_attn_workspace_bytes(None) == 0

@@ -188,19 +188,39 @@ def test_mask_free_padding_path_matches_masked_model():
     assert abs(loss_p - loss_e) < 2e-2 * abs(loss_e), (loss_e, loss_p)
 
 
-def test_float32_tensors_are_accepted_at_bf16_accuracy():
-    """Config 1 as given (fp32 tensors): accepted, computed in bf16, results returned in fp32."""
+def test_float16_tensors_are_accepted_at_bf16_accuracy():
+    """float16 tensors are rounded to bfloat16 on the way in and the results cast back."""
     import oregon_gpt_oss_patching_amd as A
-    q, k, v, sinks, d_out = E.make_inputs(1, 1, 8, 2, 256, 64, torch.float32)
+    q, k, v, sinks, d_out = E.make_inputs(1, 1, 8, 2, 256, 64, torch.float16)
     for w in (None, 32):
-        ref = E.eager_attention_grads(q, k, v, sinks, d_out, SCALE, w)
+        ref = E.eager_attention_grads(q.float(), k.float(), v.float(), sinks.float(), d_out.float(), SCALE, w)
         qd, kd, vd, sd = (t.to(DEV).requires_grad_(True) for t in (q, k, v, sinks))
         out = A.attention(qd, kd, vd, sd, SCALE, w, None)
-        assert out.dtype == torch.float32
+        assert out.dtype == torch.float16
         out.backward(d_out.to(DEV))
         for g, r in zip((out, qd.grad, kd.grad, vd.grad, sd.grad), ref):
-            assert g.dtype == torch.float32
-            assert rel_l2(g.detach().cpu(), r) < 1e-2
+            assert g.dtype == torch.float16
+            assert rel_l2(g.detach().float().cpu(), r) < 1e-2
+
+
+def test_custom_ops_are_registered_and_match_the_direct_calls():
+    """`gptoss_attn::fwd` / `gptoss_attn::bwd` are what the autograd.Function runs; they must equal
+    the direct library calls bit for bit, and their shape-only implementations must agree with
+    the real ones (torch.library.opcheck)."""
+    import oregon_gpt_oss_patching_amd as A
+    q, k, v, sinks, d_out = (t.to(DEV) for t in E.make_inputs(9, 1, 8, 2, 130, 64, torch.bfloat16))
+    o, lse = torch.ops.gptoss_attn.fwd(q, k, v, sinks, SCALE, 32, 0, None, None)
+    o2, lse2 = A.attention_forward(q, k, v, sinks, SCALE, 32)
+    assert torch.equal(o, o2) and torch.equal(lse, lse2)
+    got = torch.ops.gptoss_attn.bwd(q, k, v, sinks, o, lse, d_out, SCALE, 32, 0, None, None, True)
+    ref = A.attention_backward(q, k, v, sinks, o, lse, d_out, SCALE, 32)
+    for g, r in zip(got, ref):
+        assert torch.equal(g, r)
+    assert torch.ops.gptoss_attn.bwd(q, k, v, sinks, o, lse, d_out, SCALE, 32, 0, None, None, False)[3].numel() == 0
+    torch.library.opcheck(torch.ops.gptoss_attn.fwd.default, (q, k, v, sinks, SCALE, 32, 0, None, None),
+                          test_utils=("test_schema", "test_faketensor"))
+    torch.library.opcheck(torch.ops.gptoss_attn.bwd.default, (q, k, v, sinks, o, lse, d_out, SCALE, 32, 0, None, None, True),
+                          test_utils=("test_schema", "test_faketensor"))
 
 
 def test_packed_rows_through_the_patched_model():

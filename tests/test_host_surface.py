@@ -74,3 +74,19 @@ def test_mask_free_attention_mask_carries_lengths():
     m = sft_bench.mask_free_attention_mask(pad)
     assert m["full_attention"].tolist() == [3, 4] and m["full_attention"].dtype == torch.int32
     assert m["sliding_attention"] is m["full_attention"]
+
+
+def test_custom_ops_have_shape_only_implementations():
+    """The operators the autograd.Function calls are registered at import, and their
+    shape-only ("fake") implementations run without a GPU (meta tensors)."""
+    import oregon_gpt_oss_patching_amd.attention_kernel as ak
+    assert ak.OP_NAMESPACE == "gptoss_attn"
+    q = torch.empty(2, 8, 100, 64, dtype=torch.bfloat16, device="meta")
+    k = torch.empty(2, 2, 100, 64, dtype=torch.bfloat16, device="meta")
+    sinks = torch.empty(8, dtype=torch.bfloat16, device="meta")
+    o, lse = torch.ops.gptoss_attn.fwd(q, k, k, sinks, 0.125, 128, 0, None, None)
+    assert o.shape == (2, 100, 8, 64) and o.dtype == torch.bfloat16
+    assert lse.shape == (2, 8, 100) and lse.dtype == torch.float32
+    dq, dk, dv, ds = torch.ops.gptoss_attn.bwd(q, k, k, sinks, o, lse, o, 0.125, 128, 0, None, None, True)
+    assert dq.shape == q.shape and dk.shape == k.shape and dv.shape == k.shape and ds.shape == (8,)
+    assert torch.ops.gptoss_attn.bwd(q, k, k, None, o, lse, o, 0.125, 0, 0, None, None, False)[3].numel() == 0
