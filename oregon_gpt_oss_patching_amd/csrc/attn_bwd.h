@@ -256,25 +256,51 @@ __global__ __launch_bounds__(NW * 64, (NB == 1 ? 2 : 1)) void attn_bwd_dkdv_kern
     // Iteration `it` -> (query tile, query head).  Query tiles run from the LAST one
     // down and heads are the inner index, so every workgroup of this KV head that is
     // resident at the same time walks the same Q / dO tiles in the same order and finds
-    // them in its XCD's L2.
+    // them in its XCD's L2.  The walk is kept as running pointers (one step per request):
+    // no division or 64-bit multiplication in the loop.
+    const AsyncLaneOffsets qlane = make_async_offsets(a.qs.s, lane, w), glane = make_async_offsets(a.dos.s, lane, w);
+    int iss_h = 0, iss_i0 = (qt_hi - 1) * kTile;                      // head within the group, first row of the tile
+    const bf16 *qtile = a.q + (int64_t)b * a.qs.b + (int64_t)(g * a.r) * a.qs.h + (int64_t)iss_i0 * a.qs.s;
+    const bf16 *gtile = a.d_o + (int64_t)b * a.dos.b + (int64_t)(g * a.r) * a.dos.h + (int64_t)iss_i0 * a.dos.s;
+    int64_t stat_off = ((int64_t)b * a.H + (int64_t)g * a.r) * a.Sq + iss_i0;    // (b, head, row) of the tile's first row
+    // wavefront w copies 32 floats of lse2 (w < 2) or delta (w >= 2) per tile; 16 document starts
+    const float *stat_lane = ((w >> 1) ? a.delta : lse2) + 32 * (w & 1) + (lane & 31);
+    const int32_t *doc_lane = DOCS ? a.doc_start + (int64_t)b * a.Sq + 16 * w + (lane & 15) : nullptr;
     auto issue = [&](int it) {
         const int stage = it % NS;
-        const int hq = g * a.r + it % a.r;
-        const int i0 = (qt_hi - 1 - it / a.r) * kTile;
-        tile_async(smem[stage][0], a.q + (int64_t)b * a.qs.b + (int64_t)hq * a.qs.h, a.qs.s, i0, a.Sq, lane, w);
-        tile_async(smem[stage][1], a.d_o + (int64_t)b * a.dos.b + (int64_t)hq * a.dos.h, a.dos.s, i0, a.Sq, lane, w);
-        // row statistics: wavefront w copies 32 floats of lse2 (w < 2) or delta (w >= 2)
-        if (lane < 32) {
-            const int i = min(i0 + 32 * (w & 1) + lane, a.Sq - 1);
-            const float *src = ((w >> 1) ? a.delta : lse2) + ((int64_t)b * a.H + hq) * a.Sq + i;
-            __builtin_amdgcn_global_load_lds((glb_void_t *)src, (lds_void_t *)(&sstat[stage][w >> 1][32 * (w & 1)]), 4, 0, 0);
+        if (iss_i0 + kTile <= a.Sq) {
+            tile_async_inner(smem[stage][0], qtile, qlane, w);
+            tile_async_inner(smem[stage][1], gtile, glane, w);
+            if (lane < 32)
+                __builtin_amdgcn_global_load_lds((glb_void_t *)(stat_lane + stat_off), (lds_void_t *)(&sstat[stage][w >> 1][32 * (w & 1)]), 4, 0, 0);
+            if (DOCS && lane < 16)
+                __builtin_amdgcn_global_load_lds((glb_void_t *)(doc_lane + iss_i0), (lds_void_t *)(&sdoc[DOCS ? stage : 0][16 * w]), 4, 0, 0);
+        } else {
+            // the tile sticks out of the tensor: rows past the end re-read the last valid one
+            tile_async(smem[stage][0], qtile - (int64_t)iss_i0 * a.qs.s, a.qs.s, iss_i0, a.Sq, lane, w);
+            tile_async(smem[stage][1], gtile - (int64_t)iss_i0 * a.dos.s, a.dos.s, iss_i0, a.Sq, lane, w);
+            if (lane < 32) {
+                const int over = max(0, iss_i0 + 32 * (w & 1) + lane - (a.Sq - 1));
+                __builtin_amdgcn_global_load_lds((glb_void_t *)(stat_lane + stat_off - over), (lds_void_t *)(&sstat[stage][w >> 1][32 * (w & 1)]), 4, 0, 0);
+            }
+            if (DOCS && lane < 16) {
+                const int over = max(0, iss_i0 + 16 * w + lane - (a.Sq - 1));
+                __builtin_amdgcn_global_load_lds((glb_void_t *)(doc_lane + iss_i0 - over), (lds_void_t *)(&sdoc[DOCS ? stage : 0][16 * w]), 4, 0, 0);
+            }
         }
-        if (DOCS && lane < 16) {          // wavefront w copies the document starts of 16 rows
-            const int i = min(i0 + 16 * w + lane, a.Sq - 1);
-            const int32_t *src = a.doc_start + (int64_t)b * a.Sq + i;
-            __builtin_amdgcn_global_load_lds((glb_void_t *)src, (lds_void_t *)(&sdoc[DOCS ? stage : 0][16 * w]), 4, 0, 0);
+        ++iss_h;
+        qtile += a.qs.h;
+        gtile += a.dos.h;
+        stat_off += a.Sq;
+        if (iss_h == a.r) {
+            iss_h = 0;
+            iss_i0 -= kTile;
+            qtile -= (int64_t)a.r * a.qs.h + (int64_t)kTile * a.qs.s;
+            gtile -= (int64_t)a.r * a.dos.h + (int64_t)kTile * a.dos.s;
+            stat_off -= (int64_t)a.r * a.Sq + kTile;
         }
     };
+    int cur_h = 0, cur_i0 = (qt_hi - 1) * kTile;                      // the same walk for the tile being consumed
     // vector-memory instructions one wavefront issues per iteration: 5, or 6 with document starts
 
     // One iteration on a compile-time LDS stage, so that every fragment address is
@@ -290,7 +316,8 @@ __global__ __launch_bounds__(NW * 64, (NB == 1 ? 2 : 1)) void attn_bwd_dkdv_kern
         const uint32_t qsm = smem_base + STAGE * (2 * kStageTileBytes), gsm = qsm + kStageTileBytes;
         const uint32_t stat_lane = stat_base + STAGE * (2 * kTile * 4) + half * 16;
         const uint32_t ds_lane = doc_base + STAGE * (kTile * 4) + half * 16;
-        const int i0 = (qt_hi - 1 - it / a.r) * kTile;
+        const int i0 = cur_i0;
+        if (++cur_h == a.r) { cur_h = 0; cur_i0 -= kTile; }
         const int pos0 = a.q_offset + i0;                                    // first query position of the tile
         const int pos1 = min(a.q_offset + min(a.Sq, i0 + kTile) - 1, q_len - 1);   // last live one
         const int wj1 = min(wj0 + WK, kv_len) - 1;                           // wavefront's last live key
