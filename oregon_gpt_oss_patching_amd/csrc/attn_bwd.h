@@ -517,10 +517,23 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_bwd_dq_kernel(co
     const TileLaneOffsets lo = make_tile_offsets(lane);
     const uint32_t smem_base = lds_addr(&smem[0][0][0]);
     const int n_it = max(0, t_hi - t_lo);
+    // K / V tiles are requested in order; the pointers to the next tile's first row advance by
+    // one tile per request.  Only a tile that sticks out of the tensor takes the clamping copy.
+    const AsyncLaneOffsets klane = make_async_offsets(a.ks.s, lane, w), vlane = make_async_offsets(a.vs.s, lane, w);
+    const bf16 *ktile = kbase + (int64_t)t_lo * kTile * a.ks.s, *vtile = vbase + (int64_t)t_lo * kTile * a.vs.s;
+    int next_row0 = t_lo * kTile;
     auto issue = [&](int it) {
         const int stage = it % NS;
-        tile_async(smem[stage][0], kbase, a.ks.s, (t_lo + it) * kTile, a.Skv, lane, w);
-        tile_async(smem[stage][1], vbase, a.vs.s, (t_lo + it) * kTile, a.Skv, lane, w);
+        if (next_row0 + kTile <= a.Skv) {
+            tile_async_inner(smem[stage][0], ktile, klane, w);
+            tile_async_inner(smem[stage][1], vtile, vlane, w);
+        } else {
+            tile_async(smem[stage][0], kbase, a.ks.s, next_row0, a.Skv, lane, w);
+            tile_async(smem[stage][1], vbase, a.vs.s, next_row0, a.Skv, lane, w);
+        }
+        ktile += kTile * a.ks.s;
+        vtile += kTile * a.vs.s;
+        next_row0 += kTile;
     };
     constexpr int kLoadsPerIt = 4;
 

@@ -69,6 +69,16 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 // fmaxf costs in IEEE mode (the kernels never produce NaN: masked logits are -inf and the
 // running max is finite).
 __device__ __forceinline__ float fast_max(float a, float b) { return __builtin_amdgcn_fmed3f(a, b, INFINITY); }
+// max(x of this lane, x of lane ^ 32): v_permlane32_swap exchanges the two 32-lane halves in
+// the VALU, so the reduction does not queue behind outstanding LDS reads as a ds_bpermute would.
+// swap(a, b) returns {a.lo | b.lo, a.hi | b.hi} (low 32 lanes | high 32 lanes).
+__device__ __forceinline__ float xhalf_max(float x) {
+    typedef __attribute__((ext_vector_type(2))) unsigned u32x2_t;
+    const unsigned u = __float_as_uint(x);
+    const u32x2_t r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    const unsigned lo = r.x, hi = r.y;     // copied out first: bit-casting the vector elements in place reads element 0 twice
+    return fast_max(__uint_as_float(lo), __uint_as_float(hi));
+}
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
 // ---- staging a 64 x 64 tile: global -> registers -> LDS, NT threads --------------

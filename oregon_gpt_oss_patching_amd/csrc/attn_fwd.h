@@ -75,7 +75,7 @@ __device__ __forceinline__ void fwd_tile(uint32_t ksm, uint32_t vsm, const TileL
 #pragma unroll
         for (int i = 1; i < 16; ++i) { mx0 = fast_max(mx0, s[0][qb][i]); mx1 = fast_max(mx1, s[1][qb][i]); }
         float mx = fast_max(mx0, mx1);
-        mx = fast_max(mx, __shfl_xor(mx, 32));
+        mx = xhalf_max(mx);
         const float m_new = fast_max(m[qb], mx * c);
         if (__builtin_amdgcn_ballot_w64(m_new != m[qb]) != 0ull) {
             const float alpha = fast_exp2(m[qb] - m_new);
@@ -204,10 +204,23 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_fwd_kernel(const
     const TileLaneOffsets lo = make_tile_offsets(lane);
     const uint32_t smem_base = lds_addr(&smem[0][0][0]);
     const int n_it = max(0, t_hi - t_lo);
+    // K / V tiles are requested in order; the pointers to the next tile's first row advance by
+    // one tile per request.  Only a tile that sticks out of the tensor takes the clamping copy.
+    const AsyncLaneOffsets klane = make_async_offsets(a.ks.s, lane, w), vlane = make_async_offsets(a.vs.s, lane, w);
+    const bf16 *ktile = kbase + (int64_t)t_lo * kTile * a.ks.s, *vtile = vbase + (int64_t)t_lo * kTile * a.vs.s;
+    int next_row0 = t_lo * kTile;
     auto issue = [&](int it) {
         const int stage = it % NS;
-        tile_async(smem[stage][0], kbase, a.ks.s, (t_lo + it) * kTile, a.Skv, lane, w);
-        tile_async(smem[stage][1], vbase, a.vs.s, (t_lo + it) * kTile, a.Skv, lane, w);
+        if (next_row0 + kTile <= a.Skv) {
+            tile_async_inner(smem[stage][0], ktile, klane, w);
+            tile_async_inner(smem[stage][1], vtile, vlane, w);
+        } else {
+            tile_async(smem[stage][0], kbase, a.ks.s, next_row0, a.Skv, lane, w);
+            tile_async(smem[stage][1], vbase, a.vs.s, next_row0, a.Skv, lane, w);
+        }
+        ktile += kTile * a.ks.s;
+        vtile += kTile * a.vs.s;
+        next_row0 += kTile;
     };
     constexpr int kLoadsPerIt = 4;     // vector-memory instructions one wavefront issues per iteration
 
