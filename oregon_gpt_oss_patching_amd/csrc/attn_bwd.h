@@ -379,7 +379,7 @@ __global__ __launch_bounds__(NW * 64, (NB == 1 ? 2 : 1)) void attn_bwd_dkdv_kern
 template <bool MASKED, int NQB>
 __device__ __forceinline__ void dq_tile(uint32_t ksm, uint32_t vsm, const TileLaneOffsets &lo, const bf16x8 (&qf)[NQB][4],
                                         const bf16x8 (&gf)[NQB][4], f32x16 (&dq)[NQB][2], const float (&lse2)[NQB],
-                                        const float (&dlt)[NQB], float c, int lane, const int (&dbase)[NQB],
+                                        const float (&dlt)[NQB], const f32x16 &dseed, float c, int lane, const int (&dbase)[NQB],
                                         const unsigned (&wl)[NQB], unsigned weff, int key_lim, int wrel) {
     // wrel (masked variant only): (first query position of the wavefront) - (first key of the
     // tile); a 32-key half of the tile that no row of the wavefront can see is skipped.
@@ -387,6 +387,9 @@ __device__ __forceinline__ void dq_tile(uint32_t ksm, uint32_t vsm, const TileLa
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
         if (MASKED && ((32 * kb > wrel + 32 * NQB - 1) || (32 * kb + 31 < wrel - (int)weff + 1) || (32 * kb >= key_lim))) continue;
+        // the dP accumulators of the first query block start at -delta (dseed, the first MFMA's C
+        // operand: sixteen copies of the lane's value), so that block needs no subtraction afterwards;
+        // the register file has no room for a second such block
         f32x16 s[NQB], dp[NQB];
 #pragma unroll
         for (int qb = 0; qb < NQB; ++qb)
@@ -399,7 +402,7 @@ __device__ __forceinline__ void dq_tile(uint32_t ksm, uint32_t vsm, const TileLa
 #pragma unroll
             for (int qb = 0; qb < NQB; ++qb) {
                 s[qb] = mfma_bf16(ak, qf[qb][ks], s[qb]);
-                dp[qb] = mfma_bf16(av, gf[qb][ks], dp[qb]);
+                dp[qb] = mfma_bf16(av, gf[qb][ks], (ks == 0 && qb == 0) ? dseed : dp[qb]);
             }
         }
 #pragma unroll
@@ -412,7 +415,7 @@ __device__ __forceinline__ void dq_tile(uint32_t ksm, uint32_t vsm, const TileLa
                     const bool vis = ((unsigned)(dbase[qb] - r) < wl[qb]) & (r < key_lim);
                     pe = vis ? pe : 0.0f;
                 }
-                dp[qb][i] = pe * (dp[qb][i] + dlt[qb]);        // dlt holds -delta
+                dp[qb][i] = qb == 0 ? pe * dp[qb][i] : pe * (dp[qb][i] + dlt[qb]);        // dlt holds -delta
             }
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
@@ -508,7 +511,9 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_bwd_dq_kernel(co
     }
 
     const float c = a.scale_log2;
-    f32x16 dq[NQB][2];
+    f32x16 dq[NQB][2], dseed;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) dseed[i] = dlt[0];
 #pragma unroll
     for (int qb = 0; qb < NQB; ++qb)
 #pragma unroll
@@ -550,12 +555,12 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_bwd_dq_kernel(co
         const bool interior = (n0 + kTile - 1 <= wpos0) && (n0 > wpos1 - weff) && (n0 + kTile <= kv_len) &&
                               (a.q_offset + qw0 + WM - 1 <= wpos1) && (n0 >= ds_w1);
         if (interior) {
-            dq_tile<false, NQB>(ksm, vsm, lo, qf, gf, dq, lse2, dlt, c, lane, pq, wl, 0u, 0, 0);
+            dq_tile<false, NQB>(ksm, vsm, lo, qf, gf, dq, lse2, dlt, dseed, c, lane, pq, wl, 0u, 0, 0);
         } else {
             int dbase[NQB];
 #pragma unroll
             for (int qb = 0; qb < NQB; ++qb) dbase[qb] = pq[qb] - n0;
-            dq_tile<true, NQB>(ksm, vsm, lo, qf, gf, dq, lse2, dlt, c, lane, dbase, wl, (unsigned)weff, kv_len - n0, wpos0 - n0);
+            dq_tile<true, NQB>(ksm, vsm, lo, qf, gf, dq, lse2, dlt, dseed, c, lane, dbase, wl, (unsigned)weff, kv_len - n0, wpos0 - n0);
         }
     };
 
