@@ -499,8 +499,36 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_bwd_dq_kernel(co
         }
         lse2[qb] = 0.0f;
         dlt[qb] = 0.0f;
-        if (row_ok) {
-            const int64_t off = ((int64_t)b * a.H + head) * a.Sq + row;
+        const int64_t off = ((int64_t)b * a.H + head) * a.Sq + row;
+        if (a.fuse_delta) {
+            // No separate preprocess launch: this wavefront owns its rows, so it computes their
+            // -delta = -sum_d dO*O and lse*log2(e) itself and leaves both in the scratch buffer for
+            // the dK/dV and dSinks kernels, which then have to run after this one.  The lane holds
+            // the 16-byte chunks 2*ks + half of its row; the sums are taken in the order of
+            // attn_bwd_delta_kernel (chunk by chunk, then chunk pairs, pairs of pairs), so the
+            // values are bit-identical to that kernel's.
+            const bf16 *orow = a.o + (int64_t)b * a.os.b + (int64_t)head * a.os.h + (int64_t)row * a.os.s;
+            float t[4];
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks) {
+                u32x4 zo = {0u, 0u, 0u, 0u};
+                if (row_ok) zo = *reinterpret_cast<const u32x4 *>(orow + 16 * ks + 8 * half);
+                const bf16x8 of = as_bf16x8(zo);
+                float acc = 0.0f;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc = fmaf((float)of[j], (float)gf[qb][ks][j], acc);
+                t[ks] = xhalf_sum(acc);
+            }
+            const float dsum = (t[0] + t[1]) + (t[2] + t[3]);
+            if (row_ok) {
+                dlt[qb] = -dsum;
+                lse2[qb] = a.lse[off] * kLog2e;
+                if (half == 0 && active) {
+                    a.delta[off] = dlt[qb];
+                    a.delta[(int64_t)a.B * a.H * a.Sq + off] = lse2[qb];
+                }
+            }
+        } else if (row_ok) {
             lse2[qb] = a.delta[(int64_t)a.B * a.H * a.Sq + off];   // lse * log2(e), written by the delta kernel
             dlt[qb] = a.delta[off];                                  // -delta
         }

@@ -52,6 +52,7 @@ struct KArgs {
     int q_offset;
     float scale;
     float scale_log2;    // scale * log2(e)
+    int fuse_delta;      // dQ kernel only: compute -delta and lse*log2(e) itself and store them in the scratch
 };
 
 __device__ __forceinline__ int crow(int i, int half) { return 8 * (i >> 2) + 4 * half + (i & 3); }
@@ -78,6 +79,14 @@ __device__ __forceinline__ float xhalf_max(float x) {
     const u32x2_t r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
     const unsigned lo = r.x, hi = r.y;     // copied out first: bit-casting the vector elements in place reads element 0 twice
     return fast_max(__uint_as_float(lo), __uint_as_float(hi));
+}
+// x of this lane + x of lane ^ 32 (same exchange as xhalf_max)
+__device__ __forceinline__ float xhalf_sum(float x) {
+    typedef __attribute__((ext_vector_type(2))) unsigned u32x2_t;
+    const unsigned u = __float_as_uint(x);
+    const u32x2_t r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    const unsigned lo = r.x, hi = r.y;
+    return __uint_as_float(lo) + __uint_as_float(hi);
 }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 

@@ -185,10 +185,12 @@ int gptoss_attn_bwd_dkdv(const gptoss_attn_params *p, void *stream) {
     return launch_status();
 }
 
-int gptoss_attn_bwd_dq(const gptoss_attn_params *p, void *stream) {
+// The dQ launch; fuse_delta: the kernel also produces the row statistics (see attn_bwd_dq_kernel).
+static int launch_dq(const gptoss_attn_params *p, void *stream, int fuse_delta) {
     const int rc = gptoss_attn_validate(p, 1);
     if (rc) return rc;
-    const KArgs a = make_args(p);
+    KArgs a = make_args(p);
+    a.fuse_delta = fuse_delta;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (p->dtype == GPTOSS_ATTN_FP32) {
         hipLaunchKernelGGL(attn_f32_dq_kernel, dim3(f32_grid((int64_t)a.B * a.H * ((a.Sq + 31) / 32))), dim3(256), 0, st, a);
@@ -208,12 +210,30 @@ int gptoss_attn_bwd_dq(const gptoss_attn_params *p, void *stream) {
     return launch_status();
 }
 
+int gptoss_attn_bwd_dq(const gptoss_attn_params *p, void *stream) { return launch_dq(p, stream, 0); }
+
+// The whole backward.  bf16: the dQ kernel computes the row statistics on the way (no separate
+// pass over O and dO), then dSinks and dK/dV read them from the scratch buffer.  The results are
+// bit-identical to gptoss_attn_bwd_preprocess + gptoss_attn_bwd_dkdv + gptoss_attn_bwd_dq.
 int gptoss_attn_bwd(const gptoss_attn_params *p, void *stream) {
-    int rc = gptoss_attn_bwd_preprocess(p, stream);
+    int rc = gptoss_attn_validate(p, 1);
     if (rc) return rc;
-    rc = gptoss_attn_bwd_dkdv(p, stream);
+    if (p->dtype == GPTOSS_ATTN_FP32) {
+        rc = gptoss_attn_bwd_preprocess(p, stream);
+        if (rc) return rc;
+        rc = gptoss_attn_bwd_dkdv(p, stream);
+        if (rc) return rc;
+        return gptoss_attn_bwd_dq(p, stream);
+    }
+    rc = launch_dq(p, stream, 1);
     if (rc) return rc;
-    return gptoss_attn_bwd_dq(p, stream);
+    if (p->dsinks) {
+        const KArgs a = make_args(p);
+        hipLaunchKernelGGL(attn_bwd_dsinks_kernel, dim3((unsigned)a.H), dim3(1024), 0, static_cast<hipStream_t>(stream), a);
+        rc = launch_status();
+        if (rc) return rc;
+    }
+    return gptoss_attn_bwd_dkdv(p, stream);
 }
 
 }  // extern "C"
