@@ -150,8 +150,12 @@ int gptoss_attn_bwd_dkdv(const gptoss_attn_params *params, void *stream);
 int gptoss_attn_bwd_dq(const gptoss_attn_params *params, void *stream);
 
 /*
- * Whole backward (steps 1-3 on one stream), i.e. `_attention.backward`
- * (attention_kernel.py:276-344).
+ * Whole backward on one stream, i.e. `_attention.backward`
+ * (attention_kernel.py:276-344).  Same results, bit for bit, as steps 1-3 called
+ * one after the other.  For bf16 tensors it launches fewer kernels: the dQ
+ * kernel computes delta and lse*log2(e) for its own rows (no separate pass over
+ * O and dO), stores them in `delta`, and the dSinks and dK/dV kernels follow.
+ * Reads q,k,v,sinks,o,d_o,lse,seqlens,doc_start; writes dq,dk,dv,dsinks,delta.
  */
 int gptoss_attn_bwd(const gptoss_attn_params *params, void *stream);
 
