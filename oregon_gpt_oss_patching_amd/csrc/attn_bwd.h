@@ -12,13 +12,6 @@
 
 #include "attn_common.h"
 
-// Scheduling fence between software-pipeline phases (keeps early-issued LDS reads early).
-#ifdef GPTOSS_FENCE
-#define GPTOSS_SCHED_FENCE() __builtin_amdgcn_sched_barrier(0)
-#else
-#define GPTOSS_SCHED_FENCE()
-#endif
-
 namespace gptoss {
 
 // ---------------------------------------------------------------------------------

@@ -26,9 +26,8 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 
 constexpr int kD = 64;          // head_dim handled by these kernels
 constexpr int kTile = 64;       // rows per staged LDS tile
-constexpr int kLS = 72;         // LDS row stride in elements (64 + 8 pad: 16-byte
+constexpr int kLS = 72;         // row stride (elements) of the padded output stage (64 + 8 pad: 16-byte
                                 // reads of 8 consecutive rows fall in distinct banks)
-constexpr int kTileElems = kTile * kLS;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 
@@ -90,64 +89,8 @@ __device__ __forceinline__ float xhalf_sum(float x) {
 }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
-// ---- staging a 64 x 64 tile: global -> registers -> LDS, NT threads --------------
-// Thread t owns 16-byte chunk (t % 8) of rows (t / 8) + k * (NT / 8): eight
-// consecutive lanes read one whole 128-byte row, so global loads are fully
-// coalesced 128-bit accesses and the LDS writes of a row are contiguous.
-template <int NT>
-struct TileRegs { u32x4 v[512 / NT]; };
-
-template <int NT>
-__device__ __forceinline__ void tile_load(TileRegs<NT> &r, const bf16 *base, int64_t stride_s,
-                                          int row0, int row_end, int tid) {
-    const int c = tid & 7, rr = tid >> 3;
-#pragma unroll
-    for (int pass = 0; pass < 512 / NT; ++pass) {
-        const int row = row0 + rr + (NT / 8) * pass;
-        u32x4 z = {0u, 0u, 0u, 0u};
-        if (row < row_end) z = *reinterpret_cast<const u32x4 *>(base + (int64_t)row * stride_s + c * 8);
-        r.v[pass] = z;
-    }
-}
-
-template <int NT>
-__device__ __forceinline__ void tile_store(bf16 *lds, const TileRegs<NT> &r, int tid) {
-    const int c = tid & 7, rr = tid >> 3;
-#pragma unroll
-    for (int pass = 0; pass < 512 / NT; ++pass)
-        *reinterpret_cast<u32x4 *>(lds + (rr + (NT / 8) * pass) * kLS + c * 8) = r.v[pass];
-}
-
-// A (or B) fragment with the contraction along head_dim: lane reads
-// tile[32*blk + l32][16*ks + 8*half .. +8], one 128-bit LDS read.
-__device__ __forceinline__ bf16x8 frag_nat(const bf16 *lds, int blk, int ks, int lane) {
-    const int row = 32 * blk + (lane & 31), col = 16 * ks + 8 * (lane >> 5);
-    return as_bf16x8(*reinterpret_cast<const u32x4 *>(lds + row * kLS + col));
-}
-
-// A fragment of the TRANSPOSED tile, contraction along the tile's rows:
-// lane ends up holding tile[rows(half, slot)][32*dblk + l32] for slots 0..7 with
-//   rows(half, 4*t + e) = 32*blk + 16*u + 8*t + 4*half + e  = 32*blk + crow(8*u + 4*t + e, half),
-// i.e. exactly the rows that C registers 8*u .. 8*u+7 of row-block `blk` hold, so
-// those registers (converted to bf16) are the matching B fragment.
-// ds_read_b64_tr_b16 semantics (within each group of 16 lanes, i = lane % 16):
-//   result[i][e] = chunk[lane 4*e + i/4][i % 4], chunk[j] = the 4 halfwords at lane j's address.
-// Lane j therefore points at row (base + j/4), columns (dg + 4*(j%4)) .. +3.
-__device__ __forceinline__ bf16x8 frag_tr(const bf16 *lds, int blk, int u, int dblk, int lane) {
-    const int i = lane & 15, g16 = lane >> 4, half = g16 >> 1;
-    const int col = 32 * dblk + 16 * (g16 & 1) + 4 * (i & 3);
-    const int row = 32 * blk + 16 * u + 4 * half + (i >> 2);
-    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
-    const bf16 *p0 = lds + row * kLS + col;
-    const bf16 *p1 = p0 + 8 * kLS;
-    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(p0));
-    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(p1));
-    union { struct { s16x4 a, b; } s; bf16x8 v; } x;
-    x.s.a = lo; x.s.b = hi;
-    return x.v;
-}
-
-// B fragment from C registers 8*u .. 8*u+7 (see frag_tr).
+// B fragment from C registers 8*u .. 8*u+7: converted to bf16 they hold, in k-slot order, exactly
+// the rows that a transposed A fragment (ofrag_tr) of the same 16-row step holds.
 __device__ __forceinline__ bf16x8 cfrag(const f32x16 &c, int u) {
     bf16x8 f;
 #pragma unroll
@@ -214,28 +157,6 @@ template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
     static_assert(N >= 0 && N < 64, "vmcnt range");
     __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
-}
-
-// Fragment readers for a swizzled tile (same fragment contents as frag_nat / frag_tr).
-__device__ __forceinline__ bf16x8 sfrag_nat(const char *tile, int blk, int ks, int lane) {
-    const int row = 32 * blk + (lane & 31);
-    const int c = (2 * ks + (lane >> 5)) ^ swz(row);
-    return as_bf16x8(*reinterpret_cast<const u32x4 *>(tile + row * kRowBytes + c * 16));
-}
-
-__device__ __forceinline__ bf16x8 sfrag_tr(const char *tile, int blk, int u, int dblk, int lane) {
-    const int i = lane & 15, g16 = lane >> 4, half = g16 >> 1;
-    const int row = 32 * blk + 16 * u + 4 * half + (i >> 2);
-    const int chunk = 4 * dblk + 2 * (g16 & 1) + ((i & 3) >> 1);
-    const int sub = (i & 1) * 8;
-    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
-    const char *p0 = tile + row * kRowBytes + ((chunk ^ swz(row)) * 16) + sub;
-    const char *p1 = tile + (row + 8) * kRowBytes + ((chunk ^ swz(row + 8)) * 16) + sub;
-    s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(p0));
-    s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4 *)(p1));
-    union { struct { s16x4 a, b; } s; bf16x8 v; } x;
-    x.s.a = lo; x.s.b = hi;
-    return x.v;
 }
 
 // ---- register-cheap addressing of swizzled tiles --------------------------------
