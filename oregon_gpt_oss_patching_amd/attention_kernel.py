@@ -144,8 +144,9 @@ def attention_forward(q, k, v, sinks, sm_scale, window=None, q_offset=0, seqlens
 
 
 def attention_backward(q, k, v, sinks, o, lse, d_o, sm_scale, window=None, q_offset=0, seqlens=None,
-                       need_dsinks=True, doc_start=None):
-    """Runs the three backward kernels.  o and d_o are (B,S,H,D).
+                       need_dsinks=True, doc_start=None, split=False):
+    """Runs the backward: `gptoss_attn_bwd`, or with `split=True` the three separate entry points
+    (preprocess, dK/dV, dQ), which give the same bits.  o and d_o are (B,S,H,D).
     Returns (dq, dk, dv, dsinks_fp32_or_None)."""
     _check_inputs(q, k, v, sinks)
     q, k, v = _row_contiguous(q), _row_contiguous(k), _row_contiguous(v)
@@ -174,7 +175,9 @@ def attention_backward(q, k, v, sinks, o, lse, d_o, sm_scale, window=None, q_off
         _set(p.dv_stride, _strides_bhs(dv, "bhsd"))
         p.delta = delta.data_ptr()
         p.dsinks = dsinks.data_ptr() if dsinks is not None else None
-        _lib.call("gptoss_attn_bwd", p, _stream(q))
+        for name in (("gptoss_attn_bwd_preprocess", "gptoss_attn_bwd_dkdv", "gptoss_attn_bwd_dq") if split
+                     else ("gptoss_attn_bwd",)):
+            _lib.call(name, p, _stream(q))
     return dq, dk, dv, dsinks
 
 

@@ -279,6 +279,26 @@ def test_deterministic_bitwise(A):
         assert torch.equal(x, y)
 
 
+@pytest.mark.parametrize("b,h,g,s,w,lens,docs", [
+    (1, 64, 8, 1024, None, None, None), (1, 8, 2, 333, 32, None, None), (2, 8, 2, 200, None, [150, 77], None),
+    (1, 8, 2, 300, 128, None, [100, 120, 80]), (1, 6, 3, 130, 50, None, None),
+])
+def test_combined_backward_equals_separate_steps(A, b, h, g, s, w, lens, docs):
+    """gptoss_attn_bwd (dQ kernel computes delta and lse*log2e itself, then dSinks, dK/dV) against
+    preprocess + dK/dV + dQ called one after the other: the same bits in every output."""
+    q, k, v, sinks, d_out = (t.to(DEV) for t in E.make_inputs(900 + s, b, h, g, s, 64, torch.bfloat16))
+    doc_start = None
+    if docs is not None:
+        starts = torch.tensor([0] + list(np.cumsum(docs)[:-1]), dtype=torch.int32)
+        doc_start = torch.repeat_interleave(starts, torch.tensor(docs)).view(1, s).to(DEV)
+    o, lse = A.attention_forward(q, k, v, sinks, SCALE, w, 0, lens, doc_start)
+    one = A.attention_backward(q, k, v, sinks, o, lse, d_out, SCALE, w, 0, lens, doc_start=doc_start)
+    three = A.attention_backward(q, k, v, sinks, o, lse, d_out, SCALE, w, 0, lens, doc_start=doc_start, split=True)
+    torch.cuda.synchronize()
+    for x, y in zip(one, three):
+        assert torch.equal(x, y)
+
+
 def test_window_ge_seq_equals_full(A):
     inp = E.make_inputs(71, 1, 8, 2, 200, 64, torch.bfloat16)
     a = run_hip(A, *inp, None)
