@@ -262,3 +262,34 @@ def test_packed_rows_through_the_patched_model():
     assert rel_l2(ref_docs[:, 60:], ref_leaky[:, 60:]) > 0.1          # the two semantics really differ
     assert rel_l2(got_leaky, ref_leaky) < 3e-2
     assert rel_l2(got_docs, ref_docs) < 3e-2
+
+
+def test_hip_graph_capture_and_replay_match_eager_launches():
+    """The library allocates nothing and never synchronises, so forward + backward can be
+    captured in a HIP graph.  Three replays, with eager work and synchronisations in between,
+    must reproduce the eager launches bit for bit (the kernels are deterministic)."""
+    import oregon_gpt_oss_patching_amd as A
+    q, k, v, sinks, d_out = (t.to("cuda") for t in E.make_inputs(321, 1, 16, 4, 384, 64, torch.bfloat16))
+    for window in (None, 128):
+        o_ref, lse_ref = A.attention_forward(q, k, v, sinks, 0.125, window)
+        ref = (o_ref, lse_ref) + tuple(A.attention_backward(q, k, v, sinks, o_ref, lse_ref, d_out, 0.125, window))
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):                      # warm-up on the capture stream
+            o, lse = A.attention_forward(q, k, v, sinks, 0.125, window)
+            A.attention_backward(q, k, v, sinks, o, lse, d_out, 0.125, window)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            o, lse = A.attention_forward(q, k, v, sinks, 0.125, window)
+            outs = (o, lse) + tuple(A.attention_backward(q, k, v, sinks, o, lse, d_out, 0.125, window))
+        for _ in range(3):
+            for t in outs:
+                t.fill_(float("nan"))                      # eager work between the replays
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            for got, want in zip(outs, ref):
+                assert torch.equal(got, want)
