@@ -70,10 +70,11 @@ def main():
         o = torch.empty((B, S, H, D), dtype=q.dtype, device=dev)
         lse = torch.empty((B, H, S), dtype=torch.float32, device=dev)
         dq, dk, dv = torch.empty_like(q), torch.empty(k.shape, dtype=k.dtype, device=dev), torch.empty(k.shape, dtype=k.dtype, device=dev)
-        delta = torch.empty((2, B, H, S), dtype=torch.float32, device=dev)   # [-delta; lse*log2e]
         dsinks = torch.empty((H,), dtype=torch.float32, device=dev)
         s32 = sinks.float().contiguous()
         p = ak._base_params(q, k, v, s32, None, scale, window, 0)
+        # backward scratch ([-delta; lse*log2e], plus dK/dV partials when S is short), sized by the library
+        delta = torch.empty((_lib.load().gptoss_attn_workspace_bytes(p) // 4,), dtype=torch.float32, device=dev)
         p.o, p.lse = o.data_ptr(), lse.data_ptr()
         ak._set(p.o_stride, ak._strides_bhs(o, "bshd"))
         p.d_o = d_out.data_ptr()

@@ -26,7 +26,8 @@
  *   o, d_o       (B, Sq, H, D) by default in the caller's view, but addressed
  *                through the same (b, h, s) stride triple, so any layout works
  *   lse          (B, H, Sq) fp32 contiguous
- *   delta        fp32 scratch of 2*B*H*Sq elements: rowsum(dO*O), then lse*log2(e)
+ *   delta        fp32 scratch of gptoss_attn_workspace_bytes() bytes: -rowsum(dO*O), then
+ *                lse*log2(e), then (short sequences) partial dK/dV sums
  *   sinks, dsinks (H,) fp32;  sinks == NULL means a sink logit of 0, as in the
  *                reference (attention_kernel.py:39-42)
  *   seqlens      (B,) int32 or NULL: right-padding lengths.  Keys at or beyond
@@ -51,7 +52,7 @@
 extern "C" {
 #endif
 
-#define GPTOSS_ATTN_ABI_VERSION 2
+#define GPTOSS_ATTN_ABI_VERSION 3
 
 enum gptoss_attn_dtype {
     GPTOSS_ATTN_BF16 = 0, /* 2-byte bfloat16 tensors, bf16 MFMA products, fp32 accumulation: the fast path */
@@ -98,7 +99,7 @@ typedef struct gptoss_attn_params {
     const void *d_o;
     void *dq, *dk, *dv;
     float *dsinks;          /* optional: NULL skips the sink gradient */
-    float *delta;           /* 2*B*H*Sq fp32 scratch written by bwd_preprocess */
+    float *delta;           /* fp32 scratch of gptoss_attn_workspace_bytes() bytes */
 
     gptoss_attn_strides q_stride, k_stride, v_stride, o_stride;
     gptoss_attn_strides do_stride, dq_stride, dk_stride, dv_stride;
@@ -111,10 +112,13 @@ int gptoss_attn_version(void);
 const char *gptoss_attn_status_string(int status);
 
 /*
- * Bytes of the `delta` scratch buffer the backward entry points need for these shapes
- * (2 * B * H * Sq floats); 0 for a NULL or shapeless params.  The reference allocates its
- * counterpart itself (`delta = torch.empty_like(M)`, attention_kernel.py:303); here the caller
- * owns it.  Host-only.
+ * Bytes of the `delta` scratch buffer the backward entry points need for these shapes; 0 for a
+ * NULL or shapeless params.  Reads dtype, B, H, G, Sq, Skv and window.  The buffer holds
+ * 2 * B * H * Sq floats of row statistics and, when the problem has too few key blocks to fill the
+ * GPU (bf16, full-causal, short sequences), the fp32 partial dK / dV sums of the slices each key
+ * block is cut into.  The reference allocates its counterpart itself
+ * (`delta = torch.empty_like(M)`, attention_kernel.py:303) and accumulates dK / dV with atomics
+ * (:204,212); here the caller owns the scratch and the sums are taken in a fixed order.  Host-only.
  */
 size_t gptoss_attn_workspace_bytes(const gptoss_attn_params *params);
 

@@ -12,7 +12,7 @@ from typing import Optional
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIBRARY = os.path.join(_HERE, "libgptoss_attn.so")
 
-ABI_VERSION = 2
+ABI_VERSION = 3
 DTYPE_BF16 = 0
 DTYPE_FP32 = 1
 

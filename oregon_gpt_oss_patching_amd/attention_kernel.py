@@ -158,13 +158,11 @@ def attention_backward(q, k, v, sinks, o, lse, d_o, sm_scale, window=None, q_off
     dq = torch.empty((b, h, sq, d), dtype=q.dtype, device=q.device)
     dk = torch.empty(k.shape, dtype=k.dtype, device=q.device)
     dv = torch.empty(v.shape, dtype=v.dtype, device=q.device)
-    p0 = _lib.new_params()
-    p0.B, p0.H, p0.Sq = b, h, sq
-    delta = torch.empty((_lib.load().gptoss_attn_workspace_bytes(p0) // 4,), dtype=torch.float32,
-                        device=q.device)                                       # [-delta; lse*log2e]
     dsinks = torch.empty((h,), dtype=torch.float32, device=q.device) if need_dsinks else None
     with torch.cuda.device(q.device):
         p = _base_params(q, k, v, sinks32, sl, sm_scale, window, q_offset, ds)
+        # scratch: [-delta; lse*log2e], then the dK/dV partial sums of split key blocks (short sequences)
+        delta = torch.empty((_lib.load().gptoss_attn_workspace_bytes(p) // 4,), dtype=torch.float32, device=q.device)
         p.o, p.lse = o.data_ptr(), lse.data_ptr()
         _set(p.o_stride, _strides_bhs(o, "bshd"))
         p.d_o = d_o.data_ptr()

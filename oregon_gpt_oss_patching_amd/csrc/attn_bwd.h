@@ -189,6 +189,7 @@ __global__ __launch_bounds__(NW * 64, (NB == 1 ? 2 : 1)) void attn_bwd_dkdv_kern
     int bid = blockIdx.x;
     const int g = bid % a.G; bid /= a.G;
     const int b = bid % a.B; bid /= a.B;
+    const int part = bid % a.dkdv_parts; bid /= a.dkdv_parts;
     const int kt = bid;                                   // ascending: most work first
     const int j0 = kt * BN;                               // first key of the workgroup
     const int wj0 = j0 + WK * w;                          // first key of the wavefront
@@ -203,9 +204,15 @@ __global__ __launch_bounds__(NW * 64, (NB == 1 ? 2 : 1)) void attn_bwd_dkdv_kern
     int64_t i_hi64 = min((int64_t)a.Sq, (int64_t)q_len - a.q_offset);
     i_hi64 = min(i_hi64, (int64_t)j1 + weff - a.q_offset);
     const int i_hi = (j1 >= j0) ? (int)max((int64_t)0, i_hi64) : 0;
+    // With dkdv_parts > 1 the query tiles of the key block (walked from the last one down) are cut
+    // into dkdv_parts consecutive slices, one per workgroup; each leaves an fp32 partial sum and
+    // attn_bwd_dkdv_reduce_kernel adds them in a fixed order.
     const int qt_lo = i_lo / kTile;
-    const int qt_hi = (i_hi + kTile - 1) / kTile;
-    const int nq = max(0, qt_hi - qt_lo);
+    const int qt_all_hi = (i_hi + kTile - 1) / kTile;
+    const int nq_all = max(0, qt_all_hi - qt_lo);
+    const int slice = (nq_all + a.dkdv_parts - 1) / a.dkdv_parts;
+    const int qt_hi = qt_all_hi - part * slice;
+    const int nq = max(0, min(slice, nq_all - part * slice));
     const int n_it = nq * a.r;
 
     // K, V fragments (B operands): lane = key, slots = head_dim
@@ -349,6 +356,31 @@ __global__ __launch_bounds__(NW * 64, (NB == 1 ? 2 : 1)) void attn_bwd_dkdv_kern
         if (it + 2 < n_it) iterate(it + 2, std::integral_constant<int, 2>{});
     }
 
+    if (a.dkdv_parts > 1) {
+        // unscaled fp32 partial sums; lane = key row, register i of block dblk = column 32*dblk + crow(i, half),
+        // four consecutive columns per 16-byte store
+        const int64_t tensor = (int64_t)a.B * a.G * a.Skv * kD;
+        float *pk = a.dkdv_partial + (int64_t)part * 2 * tensor + (((int64_t)b * a.G + g) * a.Skv) * kD;
+        float *pv = pk + tensor;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            const int j = wj0 + 32 * nb + l32;
+            if (j < a.Skv) {
+#pragma unroll
+                for (int dblk = 0; dblk < 2; ++dblk)
+#pragma unroll
+                    for (int a4 = 0; a4 < 4; ++a4) {
+                        const int col = 32 * dblk + 8 * a4 + 4 * half;
+                        f32x4 xk, xv;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) { xk[e] = dk[nb][dblk][4 * a4 + e]; xv[e] = dv[nb][dblk][4 * a4 + e]; }
+                        *reinterpret_cast<f32x4 *>(pk + (int64_t)j * kD + col) = xk;
+                        *reinterpret_cast<f32x4 *>(pv + (int64_t)j * kD + col) = xv;
+                    }
+            }
+        }
+        return;
+    }
     __syncthreads();
     bf16 *stage_out = reinterpret_cast<bf16 *>(&smem[0][0][0]) + w * 32 * kLS;
 #pragma unroll
@@ -362,6 +394,40 @@ __global__ __launch_bounds__(NW * 64, (NB == 1 ? 2 : 1)) void attn_bwd_dkdv_kern
                      a.dvs.s, nvalid, lane);
         __builtin_amdgcn_wave_barrier();
     }
+}
+
+// ---------------------------------------------------------------------------------
+// Sum of the dK / dV partials of a split key block, in part order (bit-reproducible), scaled and
+// rounded to the output type.  One thread per 16-byte output chunk: (tensor, b, g, key, 8 columns).
+__global__ __launch_bounds__(256) void attn_bwd_dkdv_reduce_kernel(const KArgs a) {
+    const int64_t rows = (int64_t)a.B * a.G * a.Skv;
+    const int64_t tensor = rows * kD;
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;        // chunk index over both tensors
+    if (idx >= 2 * rows * 8) return;
+    const int which = (int)(idx / (rows * 8));                            // 0 = dK, 1 = dV
+    const int64_t rem = idx - (int64_t)which * rows * 8;
+    const int64_t row = rem >> 3;
+    const int c8 = (int)(rem & 7) * 8;
+    const float *src = a.dkdv_partial + (int64_t)which * tensor + row * kD + c8;
+    f32x4 lo = {0.0f, 0.0f, 0.0f, 0.0f}, hi = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int part = 0; part < a.dkdv_parts; ++part) {
+        const f32x4 x = *reinterpret_cast<const f32x4 *>(src + (int64_t)part * 2 * tensor);
+        const f32x4 y = *reinterpret_cast<const f32x4 *>(src + (int64_t)part * 2 * tensor + 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) { lo[e] += x[e]; hi[e] += y[e]; }
+    }
+    const float mul = which == 0 ? a.scale : 1.0f;
+    bf16x8 out;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) { out[e] = (bf16)(lo[e] * mul); out[4 + e] = (bf16)(hi[e] * mul); }
+    const int key = (int)(row % a.Skv);
+    const int bg = (int)(row / a.Skv);
+    const int g = bg % a.G, b = bg / a.G;
+    const Strides &st = which == 0 ? a.dks : a.dvs;
+    bf16 *dst = (which == 0 ? a.dk : a.dv) + (int64_t)b * st.b + (int64_t)g * st.h + (int64_t)key * st.s + c8;
+    union { bf16x8 v; u32x4 u; } cv;
+    cv.v = out;
+    *reinterpret_cast<u32x4 *>(dst) = cv.u;
 }
 
 // ---------------------------------------------------------------------------------

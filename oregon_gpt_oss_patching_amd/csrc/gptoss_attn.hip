@@ -51,6 +51,7 @@ KArgs make_args(const gptoss_attn_params *p) {
     a.q_offset = p->q_offset;
     a.scale = p->scale;
     a.scale_log2 = p->scale * kLog2e;
+    a.dkdv_parts = 1;
     return a;
 }
 
@@ -64,6 +65,24 @@ int query_blocks_for(int window) { return (window > 0 && window <= 1024) ? 1 : 2
 
 // 32-key blocks per wavefront in the dK/dV kernel
 constexpr int kDkdvNB = 1;
+constexpr int kDkdvWaves = 4;                        // wavefronts per dK/dV workgroup
+constexpr int kDkdvKeys = 32 * kDkdvNB * kDkdvWaves; // keys per dK/dV workgroup
+
+// Workgroups per key block in the dK/dV kernel.  One workgroup per (batch, KV head, 128 keys) fills
+// the 256 CUs (two workgroups each) only from S = 16384 on, and the causal triangle makes the first
+// key blocks many times longer than the last; shorter problems cut each key block's query tiles into
+// slices so that there are about a thousand workgroups, and sum the slices' fp32 partials afterwards.
+// A slice keeps at least four query tiles (sliding-window layers are never cut).
+int dkdv_parts_for(const gptoss_attn_params *p) {
+    if (p->dtype != GPTOSS_ATTN_BF16) return 1;
+    const int64_t blocks = (int64_t)p->G * p->B * ((p->Skv + kDkdvKeys - 1) / kDkdvKeys);
+    int parts = (int)(1024 / (blocks > 0 ? blocks : 1));
+    const int64_t rows_seen = p->window > 0 ? (int64_t)kDkdvKeys + p->window - 1 : (int64_t)p->Sq;
+    const int tiles = (int)((rows_seen < p->Sq ? rows_seen : p->Sq) + 63) / 64;
+    if (parts > tiles / 4) parts = tiles / 4;
+    if (parts > 8) parts = 8;
+    return parts < 1 ? 1 : parts;
+}
 
 // workgroups of four independent wavefronts for the float32 kernels
 unsigned f32_grid(int64_t waves) { return (unsigned)((waves + 3) / 4); }
@@ -121,9 +140,20 @@ int gptoss_attn_validate(const gptoss_attn_params *p, int need_bwd) {
     return GPTOSS_ATTN_OK;
 }
 
+// Bytes of the row-statistics part of the scratch (rounded up to 16 bytes); dK/dV partials follow.
+static size_t stats_bytes(const gptoss_attn_params *p) {
+    const size_t n = (size_t)2 * sizeof(float) * (size_t)p->B * (size_t)p->H * (size_t)p->Sq;
+    return (n + 15) & ~(size_t)15;
+}
+
 size_t gptoss_attn_workspace_bytes(const gptoss_attn_params *p) {
     if (!p || p->B <= 0 || p->H <= 0 || p->Sq <= 0) return 0;
-    return (size_t)2 * sizeof(float) * (size_t)p->B * (size_t)p->H * (size_t)p->Sq;
+    size_t n = stats_bytes(p);
+    if (p->G > 0 && p->Skv > 0) {
+        const int parts = dkdv_parts_for(p);
+        if (parts > 1) n += (size_t)parts * 2 * sizeof(float) * (size_t)p->B * (size_t)p->G * (size_t)p->Skv * kD;
+    }
+    return n;
 }
 
 int gptoss_attn_fwd(const gptoss_attn_params *p, void *stream) {
@@ -171,17 +201,22 @@ int gptoss_attn_bwd_preprocess(const gptoss_attn_params *p, void *stream) {
 int gptoss_attn_bwd_dkdv(const gptoss_attn_params *p, void *stream) {
     const int rc = gptoss_attn_validate(p, 1);
     if (rc) return rc;
-    const KArgs a = make_args(p);
+    KArgs a = make_args(p);
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (p->dtype == GPTOSS_ATTN_FP32) {
         hipLaunchKernelGGL(attn_f32_dkdv_kernel, dim3(f32_grid((int64_t)a.B * a.G * ((a.Skv + 31) / 32))), dim3(256), 0, st, a);
         return launch_status();
     }
-    constexpr int kWaves = 4;                       // wavefronts per workgroup
-    const int bn = 32 * kDkdvNB * kWaves;           // keys per workgroup
-    const unsigned grid = (unsigned)(a.G * a.B * ((a.Skv + bn - 1) / bn));
+    constexpr int kWaves = kDkdvWaves;
+    a.dkdv_parts = dkdv_parts_for(p);
+    a.dkdv_partial = reinterpret_cast<float *>(reinterpret_cast<char *>(p->delta) + stats_bytes(p));
+    const unsigned grid = (unsigned)(a.G * a.B * a.dkdv_parts * ((a.Skv + kDkdvKeys - 1) / kDkdvKeys));
     if (a.doc_start) hipLaunchKernelGGL((attn_bwd_dkdv_kernel<kWaves, kDkdvNB, true>), dim3(grid), dim3(64 * kWaves), 0, st, a);
     else hipLaunchKernelGGL((attn_bwd_dkdv_kernel<kWaves, kDkdvNB, false>), dim3(grid), dim3(64 * kWaves), 0, st, a);
+    int s = launch_status();
+    if (s || a.dkdv_parts == 1) return s;
+    const int64_t chunks = (int64_t)2 * a.B * a.G * a.Skv * 8;
+    hipLaunchKernelGGL(attn_bwd_dkdv_reduce_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, st, a);
     return launch_status();
 }
 

@@ -150,8 +150,19 @@ def test_workspace_bytes():
     lib = _lib.load()
     p = _valid_params()
     assert lib.gptoss_attn_workspace_bytes(ctypes.byref(p)) == 2 * 4 * 1 * 8 * 128
-    p.B, p.H, p.Sq = 4, 64, 16384
+    p.B, p.H, p.G, p.Sq, p.Skv = 4, 64, 8, 16384, 16384
     assert lib.gptoss_attn_workspace_bytes(ctypes.byref(p)) == 2 * 4 * 4 * 64 * 16384
+    # short sequences: the dK/dV kernel cuts each key block's query tiles into slices (here 4) and
+    # keeps their fp32 partial sums behind the row statistics; sliding-window layers are never cut
+    p.B, p.Sq, p.Skv = 1, 4096, 4096
+    stats = 2 * 4 * 1 * 64 * 4096
+    assert lib.gptoss_attn_workspace_bytes(ctypes.byref(p)) == stats + 4 * 2 * 4 * 1 * 8 * 4096 * 64
+    p.window = 128
+    assert lib.gptoss_attn_workspace_bytes(ctypes.byref(p)) == stats
+    p.window = 0
+    p.dtype = _lib.DTYPE_FP32
+    assert lib.gptoss_attn_workspace_bytes(ctypes.byref(p)) == stats
+    p.dtype = _lib.DTYPE_BF16
     p.Sq = 0
     assert lib.gptoss_attn_workspace_bytes(ctypes.byref(p)) == 0
     assert lib.gptoss_attn_workspace_bytes(None) == 0
