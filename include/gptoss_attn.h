@@ -26,7 +26,7 @@
  *   o, d_o       (B, Sq, H, D) by default in the caller's view, but addressed
  *                through the same (b, h, s) stride triple, so any layout works
  *   lse          (B, H, Sq) fp32 contiguous
- *   delta        fp32 scratch of gptoss_attn_workspace_bytes() bytes: -rowsum(dO*O), then
+ *   delta        fp32 scratch of gptoss_attn_workspace_bytes() bytes, 16-byte aligned: -rowsum(dO*O), then
  *                lse*log2(e), then (short sequences) partial dK/dV sums
  *   sinks, dsinks (H,) fp32;  sinks == NULL means a sink logit of 0, as in the
  *                reference (attention_kernel.py:39-42)
@@ -67,7 +67,9 @@ enum gptoss_attn_status {
     GPTOSS_ATTN_ERR_HEAD_DIM = -3,      /* D != 64 */
     GPTOSS_ATTN_ERR_HEADS = -4,         /* H <= 0, G <= 0 or H % G != 0 */
     GPTOSS_ATTN_ERR_SHAPE = -5,         /* B, Sq or Skv <= 0, window < 0, q_offset < 0, scale <= 0,
-                                           or doc_start with Sq != Skv or q_offset != 0 */
+                                           Sq + q_offset, Skv or window above 2^30, doc_start with
+                                           Sq != Skv or q_offset != 0, or a launch of more than
+                                           2^31-1 workgroups */
     GPTOSS_ATTN_ERR_DTYPE = -6,         /* dtype not in gptoss_attn_dtype */
     GPTOSS_ATTN_ERR_ALIGNMENT = -7,     /* a tensor base or stride breaks 16-byte row alignment */
     GPTOSS_ATTN_ERR_STRIDE = -8,        /* a sequence stride smaller than D */

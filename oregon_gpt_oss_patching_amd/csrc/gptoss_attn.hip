@@ -85,11 +85,25 @@ int dkdv_parts_for(const gptoss_attn_params *p) {
 }
 
 // workgroups of four independent wavefronts for the float32 kernels
-unsigned f32_grid(int64_t waves) { return (unsigned)((waves + 3) / 4); }
+int64_t f32_grid(int64_t waves) { return (waves + 3) / 4; }
 
-int launch_status() {
-    const hipError_t e = hipGetLastError();
+// One launch.  hipLaunchKernel reports this launch's own status, so an error some earlier call of the
+// thread left in the runtime's sticky state is neither reported here nor cleared.  A grid beyond the
+// x-dimension limit is refused on the host.
+template <typename Kernel>
+int launch(Kernel kernel, int64_t workgroups, int threads, hipStream_t st, const KArgs &a) {
+    if (workgroups <= 0 || workgroups > 0x7fffffff) return GPTOSS_ATTN_ERR_SHAPE;
+    void *args[] = {const_cast<KArgs *>(&a)};
+    const hipError_t e = hipLaunchKernel(reinterpret_cast<const void *>(kernel), dim3((unsigned)workgroups), dim3((unsigned)threads),
+                                         args, 0, st);
     return e == hipSuccess ? GPTOSS_ATTN_OK : static_cast<int>(e);
+}
+
+// workgroups of the forward / dQ launch: (KV head, chunk of HPB query heads, batch, query tile)
+int64_t q_outer_grid(const KArgs &a, int hpb, int qb) {
+    const int bm = 32 * qb * (4 / hpb);
+    const int n_hc = (a.r + hpb - 1) / hpb;
+    return (int64_t)a.G * n_hc * a.B * ((a.Sq + bm - 1) / bm);
 }
 
 }  // namespace
@@ -105,7 +119,7 @@ const char *gptoss_attn_status_string(int status) {
         case GPTOSS_ATTN_ERR_NULL_TENSOR: return "a required tensor pointer is NULL";
         case GPTOSS_ATTN_ERR_HEAD_DIM: return "head_dim must be 64";
         case GPTOSS_ATTN_ERR_HEADS: return "H and G must be positive and H divisible by G";
-        case GPTOSS_ATTN_ERR_SHAPE: return "B, Sq, Skv must be positive; window, q_offset non-negative; scale positive and finite; doc_start needs Sq == Skv and q_offset == 0";
+        case GPTOSS_ATTN_ERR_SHAPE: return "B, Sq, Skv must be positive; window, q_offset non-negative; positions and window at most 2^30; scale positive and finite; doc_start needs Sq == Skv and q_offset == 0; at most 2^31-1 workgroups";
         case GPTOSS_ATTN_ERR_DTYPE: return "unsupported dtype";
         case GPTOSS_ATTN_ERR_ALIGNMENT: return "tensor base or stride is not 16-byte aligned";
         case GPTOSS_ATTN_ERR_STRIDE: return "sequence stride smaller than head_dim";
@@ -121,6 +135,8 @@ int gptoss_attn_validate(const gptoss_attn_params *p, int need_bwd) {
     if (p->D != kD) return GPTOSS_ATTN_ERR_HEAD_DIM;
     if (p->H <= 0 || p->G <= 0 || p->H % p->G) return GPTOSS_ATTN_ERR_HEADS;
     if (p->B <= 0 || p->Sq <= 0 || p->Skv <= 0 || p->window < 0 || p->q_offset < 0) return GPTOSS_ATTN_ERR_SHAPE;
+    // positions are 32-bit in the kernels and +-2^30 marks "no window" / "dead row"
+    if ((int64_t)p->Sq + p->q_offset > (1 << 30) || p->Skv > (1 << 30) || p->window > (1 << 30)) return GPTOSS_ATTN_ERR_SHAPE;
     if (!(p->scale > 0.0f) || !(p->scale < 3.0e38f)) return GPTOSS_ATTN_ERR_SHAPE;
     if (p->doc_start && (p->Sq != p->Skv || p->q_offset != 0)) return GPTOSS_ATTN_ERR_SHAPE;
     const int eb = p->dtype == GPTOSS_ATTN_FP32 ? 4 : 2;
@@ -136,6 +152,7 @@ int gptoss_attn_validate(const gptoss_attn_params *p, int need_bwd) {
         if ((rc = check_tensor(p->dk, p->dk_stride, eb, p->D))) return rc;
         if ((rc = check_tensor(p->dv, p->dv_stride, eb, p->D))) return rc;
         if (!p->delta) return GPTOSS_ATTN_ERR_NULL_TENSOR;
+        if (!aligned16(p->delta)) return GPTOSS_ATTN_ERR_ALIGNMENT;   // the dK/dV partial sums use 16-byte accesses
     }
     return GPTOSS_ATTN_OK;
 }
@@ -161,22 +178,14 @@ int gptoss_attn_fwd(const gptoss_attn_params *p, void *stream) {
     if (rc) return rc;
     const KArgs a = make_args(p);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (p->dtype == GPTOSS_ATTN_FP32) {
-        hipLaunchKernelGGL(attn_f32_fwd_kernel, dim3(f32_grid((int64_t)a.B * a.H * ((a.Sq + 31) / 32))), dim3(256), 0, st, a);
-        return launch_status();
-    }
+    if (p->dtype == GPTOSS_ATTN_FP32)
+        return launch(attn_f32_fwd_kernel, f32_grid((int64_t)a.B * a.H * ((a.Sq + 31) / 32)), 256, st, a);
     const int hpb = hpb_for(a.r), qb = query_blocks_for(a.window);
-    const int bm = 32 * qb * (4 / hpb);
-    const int n_hc = (a.r + hpb - 1) / hpb;
-    const dim3 grid((unsigned)(a.G * n_hc * a.B * ((a.Sq + bm - 1) / bm))), block(256);
-#define GPTOSS_LAUNCH_FWD(HPB, QB) hipLaunchKernelGGL((attn_fwd_kernel<HPB, QB>), grid, block, 0, st, a)
-    if (qb == 2) {
-        if (hpb == 4) GPTOSS_LAUNCH_FWD(4, 2); else if (hpb == 2) GPTOSS_LAUNCH_FWD(2, 2); else GPTOSS_LAUNCH_FWD(1, 2);
-    } else {
-        if (hpb == 4) GPTOSS_LAUNCH_FWD(4, 1); else if (hpb == 2) GPTOSS_LAUNCH_FWD(2, 1); else GPTOSS_LAUNCH_FWD(1, 1);
-    }
+    const int64_t grid = q_outer_grid(a, hpb, qb);
+#define GPTOSS_LAUNCH_FWD(HPB, QB) launch(attn_fwd_kernel<HPB, QB>, grid, 256, st, a)
+    if (qb == 2) return hpb == 4 ? GPTOSS_LAUNCH_FWD(4, 2) : hpb == 2 ? GPTOSS_LAUNCH_FWD(2, 2) : GPTOSS_LAUNCH_FWD(1, 2);
+    return hpb == 4 ? GPTOSS_LAUNCH_FWD(4, 1) : hpb == 2 ? GPTOSS_LAUNCH_FWD(2, 1) : GPTOSS_LAUNCH_FWD(1, 1);
 #undef GPTOSS_LAUNCH_FWD
-    return launch_status();
 }
 
 int gptoss_attn_bwd_preprocess(const gptoss_attn_params *p, void *stream) {
@@ -185,16 +194,9 @@ int gptoss_attn_bwd_preprocess(const gptoss_attn_params *p, void *stream) {
     const KArgs a = make_args(p);
     hipStream_t st = static_cast<hipStream_t>(stream);
     const int64_t rows = (int64_t)a.B * a.H * a.Sq;
-    if (p->dtype == GPTOSS_ATTN_FP32)
-        hipLaunchKernelGGL(attn_f32_delta_kernel, dim3((unsigned)((rows + 15) / 16)), dim3(256), 0, st, a);
-    else
-        hipLaunchKernelGGL(attn_bwd_delta_kernel, dim3((unsigned)((rows + 127) / 128)), dim3(256), 0, st, a);
-    int s = launch_status();
-    if (s) return s;
-    if (a.dsinks) {
-        hipLaunchKernelGGL(attn_bwd_dsinks_kernel, dim3((unsigned)a.H), dim3(1024), 0, st, a);
-        s = launch_status();
-    }
+    int s = p->dtype == GPTOSS_ATTN_FP32 ? launch(attn_f32_delta_kernel, (rows + 15) / 16, 256, st, a)
+                                         : launch(attn_bwd_delta_kernel, (rows + 127) / 128, 256, st, a);
+    if (s == GPTOSS_ATTN_OK && a.dsinks) s = launch(attn_bwd_dsinks_kernel, a.H, 1024, st, a);
     return s;
 }
 
@@ -203,21 +205,16 @@ int gptoss_attn_bwd_dkdv(const gptoss_attn_params *p, void *stream) {
     if (rc) return rc;
     KArgs a = make_args(p);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (p->dtype == GPTOSS_ATTN_FP32) {
-        hipLaunchKernelGGL(attn_f32_dkdv_kernel, dim3(f32_grid((int64_t)a.B * a.G * ((a.Skv + 31) / 32))), dim3(256), 0, st, a);
-        return launch_status();
-    }
-    constexpr int kWaves = kDkdvWaves;
+    if (p->dtype == GPTOSS_ATTN_FP32)
+        return launch(attn_f32_dkdv_kernel, f32_grid((int64_t)a.B * a.G * ((a.Skv + 31) / 32)), 256, st, a);
     a.dkdv_parts = dkdv_parts_for(p);
     a.dkdv_partial = reinterpret_cast<float *>(reinterpret_cast<char *>(p->delta) + stats_bytes(p));
-    const unsigned grid = (unsigned)(a.G * a.B * a.dkdv_parts * ((a.Skv + kDkdvKeys - 1) / kDkdvKeys));
-    if (a.doc_start) hipLaunchKernelGGL((attn_bwd_dkdv_kernel<kWaves, kDkdvNB, true>), dim3(grid), dim3(64 * kWaves), 0, st, a);
-    else hipLaunchKernelGGL((attn_bwd_dkdv_kernel<kWaves, kDkdvNB, false>), dim3(grid), dim3(64 * kWaves), 0, st, a);
-    int s = launch_status();
+    const int64_t grid = (int64_t)a.G * a.B * a.dkdv_parts * ((a.Skv + kDkdvKeys - 1) / kDkdvKeys);
+    const int s = a.doc_start ? launch(attn_bwd_dkdv_kernel<kDkdvWaves, kDkdvNB, true>, grid, 64 * kDkdvWaves, st, a)
+                              : launch(attn_bwd_dkdv_kernel<kDkdvWaves, kDkdvNB, false>, grid, 64 * kDkdvWaves, st, a);
     if (s || a.dkdv_parts == 1) return s;
     const int64_t chunks = (int64_t)2 * a.B * a.G * a.Skv * 8;
-    hipLaunchKernelGGL(attn_bwd_dkdv_reduce_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, st, a);
-    return launch_status();
+    return launch(attn_bwd_dkdv_reduce_kernel, (chunks + 255) / 256, 256, st, a);
 }
 
 // The dQ launch; fuse_delta: the kernel also produces the row statistics (see attn_bwd_dq_kernel).
@@ -227,22 +224,14 @@ static int launch_dq(const gptoss_attn_params *p, void *stream, int fuse_delta) 
     KArgs a = make_args(p);
     a.fuse_delta = fuse_delta;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (p->dtype == GPTOSS_ATTN_FP32) {
-        hipLaunchKernelGGL(attn_f32_dq_kernel, dim3(f32_grid((int64_t)a.B * a.H * ((a.Sq + 31) / 32))), dim3(256), 0, st, a);
-        return launch_status();
-    }
+    if (p->dtype == GPTOSS_ATTN_FP32)
+        return launch(attn_f32_dq_kernel, f32_grid((int64_t)a.B * a.H * ((a.Sq + 31) / 32)), 256, st, a);
     const int hpb = hpb_for(a.r), qb = query_blocks_for(a.window);
-    const int bm = 32 * qb * (4 / hpb);
-    const int n_hc = (a.r + hpb - 1) / hpb;
-    const dim3 grid((unsigned)(a.G * n_hc * a.B * ((a.Sq + bm - 1) / bm))), block(256);
-#define GPTOSS_LAUNCH_DQ(HPB, QB) hipLaunchKernelGGL((attn_bwd_dq_kernel<HPB, QB>), grid, block, 0, st, a)
-    if (qb == 2) {
-        if (hpb == 4) GPTOSS_LAUNCH_DQ(4, 2); else if (hpb == 2) GPTOSS_LAUNCH_DQ(2, 2); else GPTOSS_LAUNCH_DQ(1, 2);
-    } else {
-        if (hpb == 4) GPTOSS_LAUNCH_DQ(4, 1); else if (hpb == 2) GPTOSS_LAUNCH_DQ(2, 1); else GPTOSS_LAUNCH_DQ(1, 1);
-    }
+    const int64_t grid = q_outer_grid(a, hpb, qb);
+#define GPTOSS_LAUNCH_DQ(HPB, QB) launch(attn_bwd_dq_kernel<HPB, QB>, grid, 256, st, a)
+    if (qb == 2) return hpb == 4 ? GPTOSS_LAUNCH_DQ(4, 2) : hpb == 2 ? GPTOSS_LAUNCH_DQ(2, 2) : GPTOSS_LAUNCH_DQ(1, 2);
+    return hpb == 4 ? GPTOSS_LAUNCH_DQ(4, 1) : hpb == 2 ? GPTOSS_LAUNCH_DQ(2, 1) : GPTOSS_LAUNCH_DQ(1, 1);
 #undef GPTOSS_LAUNCH_DQ
-    return launch_status();
 }
 
 int gptoss_attn_bwd_dq(const gptoss_attn_params *p, void *stream) { return launch_dq(p, stream, 0); }
@@ -264,8 +253,7 @@ int gptoss_attn_bwd(const gptoss_attn_params *p, void *stream) {
     if (rc) return rc;
     if (p->dsinks) {
         const KArgs a = make_args(p);
-        hipLaunchKernelGGL(attn_bwd_dsinks_kernel, dim3((unsigned)a.H), dim3(1024), 0, static_cast<hipStream_t>(stream), a);
-        rc = launch_status();
+        rc = launch(attn_bwd_dsinks_kernel, a.H, 1024, static_cast<hipStream_t>(stream), a);
         if (rc) return rc;
     }
     return gptoss_attn_bwd_dkdv(p, stream);

@@ -82,6 +82,8 @@ def test_validate_accepts_good_params():
     (lambda p: setattr(p, "Sq", 0), -5),
     (lambda p: setattr(p, "window", -1), -5),
     (lambda p: setattr(p, "q_offset", -2), -5),
+    (lambda p: setattr(p, "q_offset", 2 ** 30), -5),
+    (lambda p: setattr(p, "window", 2 ** 30 + 1), -5),
     (lambda p: setattr(p, "scale", 0.0), -5),
     (lambda p: setattr(p, "scale", float("nan")), -5),
     (lambda p: setattr(p, "q", None), -2),
@@ -89,6 +91,7 @@ def test_validate_accepts_good_params():
     (lambda p: setattr(p, "dv", None), -2),
     (lambda p: setattr(p, "delta", None), -2),
     (lambda p: setattr(p, "k", 0x1008), -7),
+    (lambda p: setattr(p, "delta", 0x1004), -7),
     (lambda p: setattr(p.v_stride, "s", 68), -7),
     (lambda p: setattr(p.v_stride, "s", 32), -8),
     (lambda p: (setattr(p, "doc_start", 0x2000), setattr(p, "q_offset", 4)), -5),
