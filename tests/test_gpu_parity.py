@@ -247,6 +247,53 @@ def test_config3_s16384_one_group_and_properties(A):
     assert torch.allclose(lhs, rhs, rtol=2e-2, atol=1.0), (lhs, rhs)
 
 
+def test_long_sequence_s65536(A):
+    """Four times the north-star length (two KV groups of eight heads): 32-bit index arithmetic
+    and the tile walks at their largest.  Window layer: one KV group exactly against the C oracle.
+    Full-causal layer: prefix equality with the S=256 problem, the last key's closed form, the
+    dSinks closed form, the dQ.Q == dK.K identity, and one middle key's dV against a direct sum
+    over the 32 731 rows that see it."""
+    s, H, G = 65536, 16, 2
+    inp = E.make_inputs(77, 1, H, G, s, 64, torch.bfloat16)
+    q, k, v, sinks, d_out = inp
+    o, lse, dq, dk, dv, ds = run_hip(A, *inp, 128)
+    g = 1
+    hs = slice(8 * g, 8 * g + 8)
+    ref = oracle_tiled(q[:, hs], k[:, g:g + 1], v[:, g:g + 1], sinks[hs], d_out[:, :, hs], 128)
+    compare_all((o[:, :, hs], lse[:, hs], dq[:, hs], dk[:, g:g + 1], dv[:, g:g + 1], ds[hs]), ref)
+
+    o, lse, dq, dk, dv, ds = run_hip(A, *inp, None)
+    for t in (o, lse, dq, dk, dv, ds):
+        assert torch.isfinite(t).all()
+    sub = tuple(t[:, :, :256].contiguous() for t in (q, k, v)) + (sinks, d_out[:, :256].contiguous())
+    ro, rlse, *_ = oracle_eager(*sub, None)
+    check("o[:256]", o[:, :256], ro)
+    assert float((lse[:, :, :256].cpu() - rlse).abs().max()) <= LSE_TOL
+    qd = q.float()[0, :, -1]
+    kk = k.float()[0].repeat_interleave(8, 0)[:, -1]
+    vv = v.float()[0].repeat_interleave(8, 0)[:, -1]
+    p_last = torch.exp((qd * kk).sum(-1) * SCALE - lse[0, :, -1].cpu())
+    go = d_out.float()[0, -1]
+    delta = (go * o.float().cpu()[0, -1]).sum(-1)
+    ds_last = p_last * ((go * vv).sum(-1) - delta)
+    check("dv[last]", dv[0, :, -1], (p_last[:, None] * go).view(G, 8, 64).sum(1))
+    check("dk[last]", dk[0, :, -1], (ds_last[:, None] * qd * SCALE).view(G, 8, 64).sum(1))
+    dl = (d_out.float() * o.float().cpu()).sum(-1).permute(0, 2, 1)
+    closed = -(torch.exp(sinks.float().view(1, -1, 1) - lse.cpu()) * dl).sum((0, 2))
+    check("dsinks", ds, closed, rel=2e-3, atol=None)
+    lhs = (dq.float() * q.to(DEV).float()).sum((0, 2, 3)).view(G, 8).sum(1)
+    rhs = (dk.float() * k.to(DEV).float()).sum((0, 2, 3))
+    assert torch.allclose(lhs, rhs, rtol=2e-2, atol=1.0), (lhs, rhs)
+    j = s // 2 + 37
+    for g_ in range(G):
+        acc = torch.zeros(64, dtype=torch.float64)
+        for h in range(8 * g_, 8 * g_ + 8):
+            sc = (q[0, h, j:].double() @ k[0, g_, j].double()) * SCALE
+            acc += torch.exp(sc - lse[0, h, j:].cpu().double()) @ d_out[0, j:, h].double()
+        err = float((dv[0, g_, j].cpu().double() - acc).abs().max())
+        assert err <= 2e-2 + 2.0 ** -8 * float(acc.abs().max()), (g_, err)
+
+
 def test_q_offset_and_longer_kv(A):
     for w in (None, 16):
         inp = E.make_inputs(31, 1, 8, 2, 40, 64, torch.bfloat16, skv=64)
