@@ -33,6 +33,18 @@ def pairs(s, w):
     return s * (s + 1) // 2 if not w or w >= s else w * s - w * (w - 1) // 2
 
 
+def device_info():
+    """What the box reports for the GPU, next to the published peak the fractions are taken against."""
+    import torch
+    pr = torch.cuda.get_device_properties(0)
+    info = {"name": pr.name, "compute_units": pr.multi_processor_count}
+    for key, attr in (("max_clock_mhz", "clock_rate"), ("hbm_gib", "total_memory")):
+        val = getattr(pr, attr, None)
+        if val is not None:
+            info[key] = round(val / 1e3) if attr == "clock_rate" else round(val / 2 ** 30)
+    return info
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -186,6 +198,7 @@ def main():
                       "speedup_vs_full": round(ms_full / ms_win, 2),
                       "speedup_target": S / 256 * 0.5},
         "kernel_ms": kern,
+        "device": device_info(),
         "roofline": {"bound": "mfma", "kernel": "attn_bwd_dkdv_kernel (full causal)",
                      "achieved": round(dkdv_tflops, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(dkdv_tflops / PEAK_BF16_TFLOPS, 4),
