@@ -72,7 +72,7 @@ enum gptoss_attn_status {
                                            2^31-1 workgroups */
     GPTOSS_ATTN_ERR_DTYPE = -6,         /* dtype not in gptoss_attn_dtype */
     GPTOSS_ATTN_ERR_ALIGNMENT = -7,     /* a tensor base or stride breaks 16-byte row alignment */
-    GPTOSS_ATTN_ERR_STRIDE = -8,        /* a sequence stride smaller than D */
+    GPTOSS_ATTN_ERR_STRIDE = -8,        /* a sequence stride smaller than D or larger than 2^24 elements */
     GPTOSS_ATTN_ERR_ABI = -9            /* struct_size does not match this library */
 };
 

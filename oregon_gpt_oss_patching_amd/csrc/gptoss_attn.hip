@@ -21,7 +21,7 @@ int check_tensor(const void *p, const gptoss_attn_strides &s, int elem_bytes, in
     if (!aligned16(p)) return GPTOSS_ATTN_ERR_ALIGNMENT;
     const int64_t per16 = 16 / elem_bytes;
     if (s.b % per16 || s.h % per16 || s.s % per16) return GPTOSS_ATTN_ERR_ALIGNMENT;
-    if (s.s < D) return GPTOSS_ATTN_ERR_STRIDE;
+    if (s.s < D || s.s > (1 << 24)) return GPTOSS_ATTN_ERR_STRIDE;   // 64 rows x stride is kept in 32 bits by the tile copies
     return GPTOSS_ATTN_OK;
 }
 
@@ -122,7 +122,7 @@ const char *gptoss_attn_status_string(int status) {
         case GPTOSS_ATTN_ERR_SHAPE: return "B, Sq, Skv must be positive; window, q_offset non-negative; positions and window at most 2^30; scale positive and finite; doc_start needs Sq == Skv and q_offset == 0; at most 2^31-1 workgroups";
         case GPTOSS_ATTN_ERR_DTYPE: return "unsupported dtype";
         case GPTOSS_ATTN_ERR_ALIGNMENT: return "tensor base or stride is not 16-byte aligned";
-        case GPTOSS_ATTN_ERR_STRIDE: return "sequence stride smaller than head_dim";
+        case GPTOSS_ATTN_ERR_STRIDE: return "sequence stride smaller than head_dim or larger than 2^24 elements";
         case GPTOSS_ATTN_ERR_ABI: return "struct_size does not match this library";
         default: return status > 0 ? "HIP runtime error (status is the hipError_t)" : "unknown status";
     }

@@ -94,6 +94,7 @@ def test_validate_accepts_good_params():
     (lambda p: setattr(p, "delta", 0x1004), -7),
     (lambda p: setattr(p.v_stride, "s", 68), -7),
     (lambda p: setattr(p.v_stride, "s", 32), -8),
+    (lambda p: setattr(p.q_stride, "s", 2 ** 24 + 64), -8),
     (lambda p: (setattr(p, "doc_start", 0x2000), setattr(p, "q_offset", 4)), -5),
     (lambda p: (setattr(p, "doc_start", 0x2000), setattr(p, "Skv", 256)), -5),
 ])
