@@ -133,8 +133,9 @@ size_t gptoss_attn_workspace_bytes(const gptoss_attn_params *params);
 int gptoss_attn_fwd(const gptoss_attn_params *params, void *stream);
 
 /*
- * Backward step 1: delta = rowsum(dO * O) (first B*H*Sq floats of `delta`) and
- * lse * log2(e) (the next B*H*Sq floats).  Replaces `_attn_bwd_precompute_D`
+ * Backward step 1: the row statistics.  The first B*H*Sq floats of `delta` receive
+ * -rowsum(dO * O) (the NEGATED row dot: it seeds the dP accumulators of the kernels that
+ * follow), the next B*H*Sq floats lse * log2(e).  Replaces `_attn_bwd_precompute_D`
  * (attention_kernel.py:102-120, 304-313) including the dO transpose copy at
  * :290.  When dsinks != NULL it also produces
  * dsinks[h] = -sum_{b,i} exp(sinks[h] - lse) * delta   (attention_kernel.py:173-176)

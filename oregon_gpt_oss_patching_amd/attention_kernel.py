@@ -45,9 +45,14 @@ def _strides_bhs(t: torch.Tensor, layout: str):
     return st[0], st[2], st[1]
 
 
-def _row_contiguous(t: torch.Tensor) -> torch.Tensor:
-    """The kernels need unit stride along head_dim and 16-byte aligned rows."""
-    if t.stride(-1) != 1 or any((s * t.element_size()) % 16 for s in t.stride()[:-1]) or t.data_ptr() % 16:
+_MAX_SEQ_STRIDE = 1 << 24   # elements; the library refuses larger sequence strides (ERR_STRIDE)
+
+
+def _row_contiguous(t: torch.Tensor, seq_dim: int = 2) -> torch.Tensor:
+    """The kernels need unit stride along head_dim, 16-byte aligned rows and a sequence stride
+    of at least head_dim and at most 2^24 elements; anything else is copied."""
+    if (t.stride(-1) != 1 or any((s * t.element_size()) % 16 for s in t.stride()[:-1]) or t.data_ptr() % 16
+            or not (t.shape[-1] <= t.stride(seq_dim) <= _MAX_SEQ_STRIDE)):
         return t.contiguous()
     return t
 
@@ -67,8 +72,36 @@ def _check_inputs(q, k, v, sinks, allow_cast=False):
         raise RuntimeError("q must be (B,H,S,D) and k, v (B,G,S_kv,D)")
     if k.shape != v.shape or q.shape[0] != k.shape[0] or q.shape[3] != k.shape[3]:
         raise RuntimeError(f"shape mismatch: q {tuple(q.shape)}, k {tuple(k.shape)}, v {tuple(v.shape)}")
-    if sinks is not None and sinks.numel() != q.shape[1]:
-        raise RuntimeError("sinks must hold one logit per query head")
+    if sinks is not None:
+        if sinks.numel() != q.shape[1]:
+            raise RuntimeError("sinks must hold one logit per query head")
+        _require_on(q, "sinks", sinks)
+    _require_on(q, "k", k)
+    _require_on(q, "v", v)
+
+
+def _require_on(q, name, t):
+    """Every tensor reaches the kernels as a raw device pointer, so it has to live on q's GPU."""
+    if not torch.is_tensor(t) or t.device != q.device:
+        where = t.device if torch.is_tensor(t) else type(t).__name__
+        raise RuntimeError(f"{name} is on {where} but q is on {q.device}: every tensor must be on q's GPU")
+
+
+def _check_saved(q, o, lse, d_o):
+    """The backward's extra tensors go to the kernels as raw pointers: refuse anything that is not
+    on q's GPU or not in the layout the kernels address, before any launch."""
+    b, h, sq, d = q.shape
+    for name, t in (("o", o), ("lse", lse), ("d_o", d_o)):
+        _require_on(q, name, t)
+    for name, t in (("o", o), ("d_o", d_o)):
+        if t.dtype != q.dtype:
+            raise RuntimeError(f"{name} has dtype {t.dtype}, expected q's dtype {q.dtype}")
+        if tuple(t.shape) != (b, sq, h, d):
+            raise RuntimeError(f"{name} must be (B, S, H, D) = {(b, sq, h, d)}, got {tuple(t.shape)}")
+    if lse.dtype != torch.float32:
+        raise RuntimeError(f"lse must be float32, got {lse.dtype}")
+    if tuple(lse.shape) != (b, h, sq):
+        raise RuntimeError(f"lse must be (B, H, S) = {(b, h, sq)}, got {tuple(lse.shape)}")
 
 
 def _base_params(q, k, v, sinks32, seqlens, scale, window, q_offset, doc_start=None):
@@ -149,8 +182,10 @@ def attention_backward(q, k, v, sinks, o, lse, d_o, sm_scale, window=None, q_off
     (preprocess, dK/dV, dQ), which give the same bits.  o and d_o are (B,S,H,D).
     Returns (dq, dk, dv, dsinks_fp32_or_None)."""
     _check_inputs(q, k, v, sinks)
+    _check_saved(q, o, lse, d_o)
     q, k, v = _row_contiguous(q), _row_contiguous(k), _row_contiguous(v)
-    o, d_o = _row_contiguous(o), _row_contiguous(d_o)
+    o, d_o = _row_contiguous(o, 1), _row_contiguous(d_o, 1)
+    lse = lse.contiguous()
     b, h, sq, d = q.shape
     sinks32 = None if sinks is None else sinks.detach().to(torch.float32).contiguous()
     sl = _prep_seqlens(seqlens, q.device, b)

@@ -41,6 +41,41 @@ def test_cpu_tensors_fail_loudly():
         A.triton_flash_attention(mod, q, k, k, None, 0.125)
 
 
+def test_backward_tensors_are_checked_before_any_launch():
+    """o, lse, d_o and sinks reach the kernels as raw pointers: a tensor on another device, of
+    another dtype or shape has to raise on the host (meta tensors stand in for the GPU here)."""
+    q = torch.empty(2, 8, 100, 64, dtype=torch.bfloat16, device="meta")
+    o = torch.empty(2, 100, 8, 64, dtype=torch.bfloat16, device="meta")
+    lse = torch.empty(2, 8, 100, dtype=torch.float32, device="meta")
+    ak._check_saved(q, o, lse, o)                                   # the good case passes
+    with pytest.raises(RuntimeError, match="lse is on cpu"):
+        ak._check_saved(q, o, torch.empty(2, 8, 100), o)
+    with pytest.raises(RuntimeError, match="d_o is on cpu"):
+        ak._check_saved(q, o, lse, torch.empty(2, 100, 8, 64, dtype=torch.bfloat16))
+    with pytest.raises(RuntimeError, match="lse must be float32"):
+        ak._check_saved(q, o, lse.to(torch.bfloat16), o)
+    with pytest.raises(RuntimeError, match=r"lse must be \(B, H, S\)"):
+        ak._check_saved(q, o, lse.transpose(1, 2), o)
+    with pytest.raises(RuntimeError, match="d_o has dtype"):
+        ak._check_saved(q, o, lse, o.to(torch.float32))
+    with pytest.raises(RuntimeError, match=r"o must be \(B, S, H, D\)"):
+        ak._check_saved(q, o.transpose(1, 2), lse, o)
+    with pytest.raises(RuntimeError, match="sinks is on cpu"):
+        ak._require_on(q, "sinks", torch.zeros(8))
+
+
+def test_row_contiguous_copies_what_the_library_would_refuse():
+    base = torch.zeros(1, 4, 6, 64, dtype=torch.bfloat16)
+    assert ak._row_contiguous(base) is base
+    assert ak._row_contiguous(base[..., ::2]).is_contiguous()              # head_dim stride 2
+    wide = torch.zeros(1, 4, 6, 4, 64, dtype=torch.bfloat16)[:, :, :, 0]    # fine: stride 256
+    assert ak._row_contiguous(wide) is wide
+    overlapped = torch.zeros(1, 4, 1, 64, dtype=torch.bfloat16).expand(1, 4, 6, 64)   # sequence stride 0 < head_dim
+    assert ak._row_contiguous(overlapped).stride(2) == 64
+    bshd = torch.zeros(1, 6, 4, 64, dtype=torch.bfloat16)
+    assert ak._row_contiguous(bshd, 1) is bshd
+
+
 def test_stride_helper_layouts():
     t = torch.empty(2, 5, 3, 64)              # (B, S, H, D)
     assert ak._strides_bhs(t, "bshd") == (5 * 3 * 64, 64, 3 * 64)
