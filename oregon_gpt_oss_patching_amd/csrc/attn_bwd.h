@@ -491,7 +491,7 @@ __device__ __forceinline__ void dq_tile(uint32_t ksm, uint32_t vsm, const TileLa
     }
 }
 
-template <int HPB, int NQB>
+template <int HPB, int NQB, bool FUSE_DELTA>   // FUSE_DELTA: also produce the row statistics of the wavefront's own rows
 __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_bwd_dq_kernel(const KArgs a) {
     constexpr int QSUB = 4 / HPB;
     constexpr int WM = 32 * NQB;
@@ -559,7 +559,7 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_bwd_dq_kernel(co
         lse2[qb] = 0.0f;
         dlt[qb] = 0.0f;
         const int64_t off = ((int64_t)b * a.H + head) * a.Sq + row;
-        if (a.fuse_delta) {
+        if constexpr (FUSE_DELTA) {
             // No separate preprocess launch: this wavefront owns its rows, so it computes their
             // -delta = -sum_d dO*O and lse*log2(e) itself and leaves both in the scratch buffer for
             // the dK/dV and dSinks kernels, which then have to run after this one.  The lane holds

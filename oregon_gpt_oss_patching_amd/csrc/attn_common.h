@@ -51,7 +51,6 @@ struct KArgs {
     int q_offset;
     float scale;
     float scale_log2;    // scale * log2(e)
-    int fuse_delta;      // dQ kernel only: compute -delta and lse*log2(e) itself and store them in the scratch
     int dkdv_parts;      // dK/dV kernel: workgroups that share one key block, each taking a slice of its query tiles
     float *dkdv_partial; // dkdv_parts > 1: fp32 partial sums, [part][dK, dV][B][G][Skv][64]
 };

@@ -221,14 +221,14 @@ int gptoss_attn_bwd_dkdv(const gptoss_attn_params *p, void *stream) {
 static int launch_dq(const gptoss_attn_params *p, void *stream, int fuse_delta) {
     const int rc = gptoss_attn_validate(p, 1);
     if (rc) return rc;
-    KArgs a = make_args(p);
-    a.fuse_delta = fuse_delta;
+    const KArgs a = make_args(p);
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (p->dtype == GPTOSS_ATTN_FP32)
         return launch(attn_f32_dq_kernel, f32_grid((int64_t)a.B * a.H * ((a.Sq + 31) / 32)), 256, st, a);
     const int hpb = hpb_for(a.r), qb = query_blocks_for(a.window);
     const int64_t grid = q_outer_grid(a, hpb, qb);
-#define GPTOSS_LAUNCH_DQ(HPB, QB) launch(attn_bwd_dq_kernel<HPB, QB>, grid, 256, st, a)
+#define GPTOSS_LAUNCH_DQ(HPB, QB) \
+    (fuse_delta ? launch(attn_bwd_dq_kernel<HPB, QB, true>, grid, 256, st, a) : launch(attn_bwd_dq_kernel<HPB, QB, false>, grid, 256, st, a))
     if (qb == 2) return hpb == 4 ? GPTOSS_LAUNCH_DQ(4, 2) : hpb == 2 ? GPTOSS_LAUNCH_DQ(2, 2) : GPTOSS_LAUNCH_DQ(1, 2);
     return hpb == 4 ? GPTOSS_LAUNCH_DQ(4, 1) : hpb == 2 ? GPTOSS_LAUNCH_DQ(2, 1) : GPTOSS_LAUNCH_DQ(1, 1);
 #undef GPTOSS_LAUNCH_DQ

@@ -247,6 +247,66 @@ def test_config3_s16384_one_group_and_properties(A):
     assert torch.allclose(lhs, rhs, rtol=2e-2, atol=1.0), (lhs, rhs)
 
 
+def _fp64_oracle_on_device(inp, window, heads_per_call=4):
+    """The eager oracle (forward, logsumexp, autograd backward) evaluated in float64 with plain torch
+    operators on the GPU, a few query heads of one KV head at a time (an S x S float64 matrix per
+    head is 2.1 GB at S = 16384, far too slow on the host cores and far too large for all 64 heads at once).
+    The kernels under test take no part in it."""
+    q, k, v, sinks, d_out = (t.to(DEV).double() for t in inp)
+    b, h, s, d = q.shape
+    g = k.shape[1]
+    r = h // g
+    o = torch.empty(b, s, h, d, dtype=torch.float64, device=DEV)
+    lse = torch.empty(b, h, s, dtype=torch.float64, device=DEV)
+    dq = torch.empty_like(q)
+    dk = torch.zeros_like(k)
+    dv = torch.zeros_like(v)
+    ds = torch.empty(h, dtype=torch.float64, device=DEV)
+    for h0 in range(0, h, heads_per_call):
+        hs = slice(h0, h0 + heads_per_call)
+        kv = h0 // r
+        assert (h0 + heads_per_call - 1) // r == kv
+        args = (q[:, hs], k[:, kv:kv + 1], v[:, kv:kv + 1], sinks[hs])
+        o_, dq_, dk_, dv_, ds_ = E.eager_attention_grads(*args, d_out[:, :, hs], SCALE, window)
+        o[:, :, hs], dq[:, hs], ds[hs] = o_, dq_, ds_
+        dk[:, kv:kv + 1] += dk_
+        dv[:, kv:kv + 1] += dv_
+        lse[:, hs] = E.logsumexp_rows(args[0], args[1], args[3], SCALE, window)
+        del o_, dq_, dk_, dv_, ds_
+    return tuple(t.cpu() for t in (o, lse, dq, dk, dv, ds))
+
+
+def test_config3_s16384_full_causal_every_element(A):
+    """The headline workload itself (B=1, S=16384, 64 query heads over 8 KV heads, full causal):
+    every element of O, lse, dQ, dK, dV and dSinks against the float64 eager oracle, and a sample
+    of rows recomputed on the host from the formulas alone (reference attention_kernel.py:60-98 for
+    O and lse, :199-217 for dQ) so that the check does not rest on the device's BLAS either."""
+    s = 16384
+    inp = E.make_inputs(3, 1, 64, 8, s, 64, torch.bfloat16)
+    q, k, v, sinks, d_out = inp
+    got = run_hip(A, *inp, None)
+    ref = _fp64_oracle_on_device(inp, None)
+    compare_all(got, ref)
+    o, lse, dq, dk, dv, ds = (t.detach().cpu() for t in got)
+    gen = torch.Generator().manual_seed(5)
+    rows = [0, 63, 64, 127, 8191, 8192, 16320, 16383] + torch.randint(0, s, (8,), generator=gen).tolist()
+    for hh in (0, 7, 29, 56, 63):
+        g = hh // 8
+        qh, kh, vh, gh = q[0, hh].double(), k[0, g].double(), v[0, g].double(), d_out[0, :, hh].double()
+        for i in rows:
+            sc = (kh[:i + 1] @ qh[i]) * SCALE
+            m = max(float(sc.max()), float(sinks[hh]))
+            z = torch.exp(sc - m).sum() + torch.exp(sinks[hh].double() - m)
+            lse_i = m + torch.log(z)
+            p = torch.exp(sc - lse_i)
+            o_i = p @ vh[:i + 1]
+            d_s = p * (vh[:i + 1] @ gh[i] - (gh[i] * o_i).sum())
+            dq_i = (d_s @ kh[:i + 1]) * SCALE
+            assert abs(float(lse[0, hh, i]) - float(lse_i)) <= LSE_TOL, (hh, i)
+            check(f"o[{hh},{i}]", o[0, i, hh], o_i.float(), rel=2e-2)
+            check(f"dq[{hh},{i}]", dq[0, hh, i], dq_i.float(), rel=2e-2)
+
+
 def test_long_sequence_s65536(A):
     """Four times the north-star length (two KV groups of eight heads): 32-bit index arithmetic
     and the tile walks at their largest.  Window layer: one KV group exactly against the C oracle.
