@@ -73,8 +73,13 @@ enum gptoss_attn_status {
     GPTOSS_ATTN_ERR_DTYPE = -6,         /* dtype not in gptoss_attn_dtype */
     GPTOSS_ATTN_ERR_ALIGNMENT = -7,     /* a tensor base or stride breaks 16-byte row alignment */
     GPTOSS_ATTN_ERR_STRIDE = -8,        /* a sequence stride smaller than D or larger than 2^24 elements */
-    GPTOSS_ATTN_ERR_ABI = -9            /* struct_size does not match this library */
+    GPTOSS_ATTN_ERR_ABI = -9,           /* struct_size does not match this library */
+    GPTOSS_ATTN_ERR_WORKSPACE = -10     /* gptoss_attn_bwd_static: 2*B*H*Sq floats do not fit the built-in scratch */
 };
+
+/* Size of the device array gptoss_attn_bwd_static keeps its row statistics in: 2*B*H*Sq floats must
+ * fit, i.e. B*H*Sq <= 2 097 152 rows (the 64-head layer at S = 16384 is 1 048 576 rows per batch row). */
+#define GPTOSS_ATTN_STATIC_SCRATCH_BYTES (16u << 20)
 
 /* (batch, head, sequence) strides in elements. */
 typedef struct gptoss_attn_strides {
@@ -165,6 +170,27 @@ int gptoss_attn_bwd_dq(const gptoss_attn_params *params, void *stream);
  * Reads q,k,v,sinks,o,d_o,lse,seqlens,doc_start; writes dq,dk,dv,dsinks,delta.
  */
 int gptoss_attn_bwd(const gptoss_attn_params *params, void *stream);
+
+/*
+ * The whole backward without any workspace from the caller and without any allocation: a variant
+ * of gptoss_attn_bwd whose scratch (the row statistics -rowsum(dO*O) and lse*log2(e)) is an array
+ * of GPTOSS_ATTN_STATIC_SCRATCH_BYTES that is part of the library's device image.  It has no
+ * counterpart in the reference (whose backward allocates `delta` and zero-filled dk/dv/dsinks with
+ * torch, attention_kernel.py:296-303); it is for callers that cannot allocate: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  `params->delta` is ignored (may be
+ * NULL); inputs and outputs are still the caller's.  Problems with B*H*Sq above 2 097 152 rows are
+ * refused with GPTOSS_ATTN_ERR_WORKSPACE before anything is launched.  Key blocks are never cut
+ * into slices here (that needs a large scratch), so short full-causal bf16 problems run slower than
+ * through gptoss_attn_bwd and their dK/dV may differ from it in the last bit (another summation
+ * order); everything else is bit-identical.  Every call on one GPU uses that GPU's single array:
+ * calls that overlap on one GPU (two streams, two threads) race; calls on one stream do not, and
+ * nothing needs clearing between calls (every value read was written earlier in the same call).
+ * The array stays resident on every GPU the library has run on until the process ends.
+ */
+int gptoss_attn_bwd_static(const gptoss_attn_params *params, void *stream);
+
+/* GPTOSS_ATTN_STATIC_SCRATCH_BYTES of the loaded library.  Host-only. */
+size_t gptoss_attn_static_scratch_bytes(void);
 
 /*
  * Host-only argument check used by every entry point; `need_bwd` != 0 also

@@ -26,6 +26,8 @@ EXPORTS = (
     "gptoss_attn_bwd_dkdv",
     "gptoss_attn_bwd_dq",
     "gptoss_attn_bwd",
+    "gptoss_attn_bwd_static",
+    "gptoss_attn_static_scratch_bytes",
 )
 
 
@@ -86,8 +88,10 @@ def load() -> ctypes.CDLL:
         lib.gptoss_attn_validate.argtypes = [ctypes.POINTER(Params), ctypes.c_int]
         lib.gptoss_attn_workspace_bytes.restype = ctypes.c_size_t
         lib.gptoss_attn_workspace_bytes.argtypes = [ctypes.POINTER(Params)]
+        lib.gptoss_attn_static_scratch_bytes.restype = ctypes.c_size_t
+        lib.gptoss_attn_static_scratch_bytes.argtypes = []
         for name in ("gptoss_attn_fwd", "gptoss_attn_bwd_preprocess", "gptoss_attn_bwd_dkdv",
-                     "gptoss_attn_bwd_dq", "gptoss_attn_bwd"):
+                     "gptoss_attn_bwd_dq", "gptoss_attn_bwd", "gptoss_attn_bwd_static"):
             fn = getattr(lib, name)
             fn.restype = ctypes.c_int
             fn.argtypes = [ctypes.POINTER(Params), ctypes.c_void_p]

@@ -3,6 +3,8 @@
 // No torch headers, no allocation, no global mutable state.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include "../../include/gptoss_attn.h"
 #include "attn_bwd.h"
 #include "attn_common.h"
@@ -124,6 +126,7 @@ const char *gptoss_attn_status_string(int status) {
         case GPTOSS_ATTN_ERR_ALIGNMENT: return "tensor base or stride is not 16-byte aligned";
         case GPTOSS_ATTN_ERR_STRIDE: return "sequence stride smaller than head_dim or larger than 2^24 elements";
         case GPTOSS_ATTN_ERR_ABI: return "struct_size does not match this library";
+        case GPTOSS_ATTN_ERR_WORKSPACE: return "the problem needs more scratch than the library's built-in array holds (gptoss_attn_static_scratch_bytes)";
         default: return status > 0 ? "HIP runtime error (status is the hipError_t)" : "unknown status";
     }
 }
@@ -200,14 +203,16 @@ int gptoss_attn_bwd_preprocess(const gptoss_attn_params *p, void *stream) {
     return s;
 }
 
-int gptoss_attn_bwd_dkdv(const gptoss_attn_params *p, void *stream) {
+// The dK/dV launch (and the sum of the partials when key blocks are cut).  whole_blocks: never cut a
+// key block, so that nothing beyond the row statistics is kept in the scratch.
+static int launch_dkdv(const gptoss_attn_params *p, void *stream, bool whole_blocks) {
     const int rc = gptoss_attn_validate(p, 1);
     if (rc) return rc;
     KArgs a = make_args(p);
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (p->dtype == GPTOSS_ATTN_FP32)
         return launch(attn_f32_dkdv_kernel, f32_grid((int64_t)a.B * a.G * ((a.Skv + 31) / 32)), 256, st, a);
-    a.dkdv_parts = dkdv_parts_for(p);
+    a.dkdv_parts = whole_blocks ? 1 : dkdv_parts_for(p);
     a.dkdv_partial = reinterpret_cast<float *>(reinterpret_cast<char *>(p->delta) + stats_bytes(p));
     const int64_t grid = (int64_t)a.G * a.B * a.dkdv_parts * ((a.Skv + kDkdvKeys - 1) / kDkdvKeys);
     const int s = a.doc_start ? launch(attn_bwd_dkdv_kernel<kDkdvWaves, kDkdvNB, true>, grid, 64 * kDkdvWaves, st, a)
@@ -216,6 +221,8 @@ int gptoss_attn_bwd_dkdv(const gptoss_attn_params *p, void *stream) {
     const int64_t chunks = (int64_t)2 * a.B * a.G * a.Skv * 8;
     return launch(attn_bwd_dkdv_reduce_kernel, (chunks + 255) / 256, 256, st, a);
 }
+
+int gptoss_attn_bwd_dkdv(const gptoss_attn_params *p, void *stream) { return launch_dkdv(p, stream, false); }
 
 // The dQ launch; fuse_delta: the kernel also produces the row statistics (see attn_bwd_dq_kernel).
 static int launch_dq(const gptoss_attn_params *p, void *stream, int fuse_delta) {
@@ -239,13 +246,13 @@ int gptoss_attn_bwd_dq(const gptoss_attn_params *p, void *stream) { return launc
 // The whole backward.  bf16: the dQ kernel computes the row statistics on the way (no separate
 // pass over O and dO), then dSinks and dK/dV read them from the scratch buffer.  The results are
 // bit-identical to gptoss_attn_bwd_preprocess + gptoss_attn_bwd_dkdv + gptoss_attn_bwd_dq.
-int gptoss_attn_bwd(const gptoss_attn_params *p, void *stream) {
+static int bwd_all(const gptoss_attn_params *p, void *stream, bool whole_blocks) {
     int rc = gptoss_attn_validate(p, 1);
     if (rc) return rc;
     if (p->dtype == GPTOSS_ATTN_FP32) {
         rc = gptoss_attn_bwd_preprocess(p, stream);
         if (rc) return rc;
-        rc = gptoss_attn_bwd_dkdv(p, stream);
+        rc = launch_dkdv(p, stream, whole_blocks);
         if (rc) return rc;
         return gptoss_attn_bwd_dq(p, stream);
     }
@@ -256,7 +263,53 @@ int gptoss_attn_bwd(const gptoss_attn_params *p, void *stream) {
         rc = launch(attn_bwd_dsinks_kernel, a.H, 1024, static_cast<hipStream_t>(stream), a);
         if (rc) return rc;
     }
-    return gptoss_attn_bwd_dkdv(p, stream);
+    return launch_dkdv(p, stream, whole_blocks);
+}
+
+int gptoss_attn_bwd(const gptoss_attn_params *p, void *stream) { return bwd_all(p, stream, false); }
+
+// ---- the backward for callers that cannot allocate ------------------------------------------
+// Same kernels as gptoss_attn_bwd; the row statistics live in a device array that is part of the
+// library image instead of a caller-provided workspace.  Each GPU has its own copy of the array
+// at its own address, looked up once per device.
+namespace {
+constexpr size_t kStaticScratchBytes = GPTOSS_ATTN_STATIC_SCRATCH_BYTES;
+constexpr int kMaxDevices = 64;
+}
+static __device__ __align__(256) float scratch[kStaticScratchBytes / sizeof(float)];
+static std::atomic<float *> scratch_ptr[kMaxDevices];     // device address of `scratch`, per device; NULL = not looked up yet
+
+static int static_scratch(float **out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return static_cast<int>(e);
+    if (dev < 0 || dev >= kMaxDevices) return GPTOSS_ATTN_ERR_WORKSPACE;
+    float *ptr = scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!ptr) {
+        // with the device current, the symbol resolves to this device's copy; two threads racing
+        // here look up the same address
+        e = hipGetSymbolAddress(reinterpret_cast<void **>(&ptr), HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return static_cast<int>(e);
+        if (!ptr) return GPTOSS_ATTN_ERR_WORKSPACE;
+        scratch_ptr[dev].store(ptr, std::memory_order_release);
+    }
+    *out = ptr;
+    return GPTOSS_ATTN_OK;
+}
+
+size_t gptoss_attn_static_scratch_bytes(void) { return kStaticScratchBytes; }
+
+int gptoss_attn_bwd_static(const gptoss_attn_params *p, void *stream) {
+    if (!p) return GPTOSS_ATTN_ERR_NULL_PARAMS;
+    if (p->struct_size != sizeof(gptoss_attn_params)) return GPTOSS_ATTN_ERR_ABI;
+    gptoss_attn_params q = *p;
+    q.delta = reinterpret_cast<float *>(static_cast<uintptr_t>(256));   // stands in for the scratch while the other arguments are checked
+    int rc = gptoss_attn_validate(&q, 1);
+    if (rc) return rc;
+    if (stats_bytes(&q) > kStaticScratchBytes) return GPTOSS_ATTN_ERR_WORKSPACE;
+    rc = static_scratch(&q.delta);
+    if (rc) return rc;
+    return bwd_all(&q, stream, true);
 }
 
 }  // extern "C"
