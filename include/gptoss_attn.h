@@ -163,10 +163,17 @@ int gptoss_attn_bwd_dq(const gptoss_attn_params *params, void *stream);
 
 /*
  * Whole backward on one stream, i.e. `_attention.backward`
- * (attention_kernel.py:276-344).  Same results, bit for bit, as steps 1-3 called
- * one after the other.  For bf16 tensors it launches fewer kernels: the dQ
- * kernel computes delta and lse*log2(e) for its own rows (no separate pass over
- * O and dO), stores them in `delta`, and the dSinks and dK/dV kernels follow.
+ * (attention_kernel.py:276-344).  bf16 tensors take one of two routes:
+ *   - sliding-window layers with window <= 128, Sq == Skv, q_offset == 0, no doc_start and
+ *     2..64 query heads per KV head: ONE kernel that reads q, k, v, o, d_o once and produces dq,
+ *     dk, dv and the dsinks terms from five matrix products per (query tile, key tile) pair
+ *     (`_attn_bwd`'s own five dots, attention_kernel.py:199-217), the row statistics formed on
+ *     the way; `delta` only holds a few dsinks partial sums.  Same values as steps 1-3 up to the
+ *     order of the fp32 sums (differences in the last bf16 bit);
+ *   - everything else: the dQ kernel computes delta and lse*log2(e) for its own rows (no
+ *     separate pass over O and dO), stores them in `delta`, and the dSinks and dK/dV kernels
+ *     follow: the same bits as steps 1-3 called one after the other.
+ * Both routes are free of atomics and bit-reproducible from run to run.
  * Reads q,k,v,sinks,o,d_o,lse,seqlens,doc_start; writes dq,dk,dv,dsinks,delta.
  */
 int gptoss_attn_bwd(const gptoss_attn_params *params, void *stream);
@@ -182,7 +189,7 @@ int gptoss_attn_bwd(const gptoss_attn_params *params, void *stream);
  * refused with GPTOSS_ATTN_ERR_WORKSPACE before anything is launched.  Key blocks are never cut
  * into slices here (that needs a large scratch), so short full-causal bf16 problems run slower than
  * through gptoss_attn_bwd and their dK/dV may differ from it in the last bit (another summation
- * order); everything else is bit-identical.  Every call on one GPU uses that GPU's single array:
+ * order); everything else is bit-identical (sliding-window layers take the same single-pass kernel).  Every call on one GPU uses that GPU's single array:
  * calls that overlap on one GPU (two streams, two threads) race; calls on one stream do not, and
  * nothing needs clearing between calls (every value read was written earlier in the same call).
  * The array stays resident on every GPU the library has run on until the process ends.

@@ -80,6 +80,33 @@ __global__ __launch_bounds__(1024) void attn_bwd_dsinks_kernel(const KArgs a) {
 }
 
 // ---------------------------------------------------------------------------------
+// dS exchange through LDS (fused backward).  The dS tile is key-major: key row r of the
+// workgroup occupies 128 bytes (64 query-row columns in bf16), chunk-swizzled by swz(r).
+// A lane of an owner wavefront (key row r, half = lane / 32) holds, per 16-row step u of the
+// 32-row block qb, the B fragment dsf: elements 0..3 are rows 16u + 4*half + 0..3, elements 4..7
+// rows 16u + 8 + 4*half + 0..3, i.e. two 8-byte pieces in the logical chunks 4*qb + 2*u and
+// 4*qb + 2*u + 1 of its key row, at byte 8*half of the chunk.  With the row's swizzle folded into
+// the base address the chunk selection is one XOR with an immediate.
+__device__ __forceinline__ uint32_t ds_store_addr(uint32_t tile, int keyrow, int half) {
+    return tile + keyrow * kRowBytes + (swz(keyrow) << 4) + 8 * half;
+}
+__device__ __forceinline__ void ds_store(uint32_t base, int qb, int u, const bf16x8 dsf) {
+    typedef __attribute__((address_space(3))) bf16x4 lds_bf16x4;
+    bf16x4 p0, p1;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) { p0[e] = dsf[e]; p1[e] = dsf[4 + e]; }
+    *reinterpret_cast<lds_bf16x4 *>((uintptr_t)(base ^ ((4 * qb + 2 * u) << 4))) = p0;
+    *reinterpret_cast<lds_bf16x4 *>((uintptr_t)(base ^ ((4 * qb + 2 * u + 1) << 4))) = p1;
+}
+__device__ __forceinline__ void ds_store_zero(uint32_t base, int qb) {
+    bf16x8 z;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) z[e] = (bf16)0.0f;
+    ds_store(base, qb, 0, z);
+    ds_store(base, qb, 1, z);
+}
+
+// ---------------------------------------------------------------------------------
 // dK, dV.  Workgroup = NW wavefronts x 64 keys of KV head g, batch b.  The K and V
 // rows of a wavefront stay in registers as MFMA B operands (two 32-key blocks, so
 // every Q / dO fragment fetched from LDS feeds two MFMAs).  The loop streams
@@ -95,12 +122,18 @@ __global__ __launch_bounds__(1024) void attn_bwd_dsinks_kernel(const KArgs a) {
 // lane's key), or a huge negative number for a dead key, so that pair (row r, key)
 // is visible iff 0 <= dbase + r < weff, tested with one unsigned compare; rows at
 // or beyond `row_lim` (relative to the tile) do not exist.
-template <bool MASKED, bool DOCS, int NB>
+// STORE_DS (needs NB == 1): the bf16 dS values of the tile are also written to LDS, key-major: the
+// lane's key row starts at ds_out (which already holds the row's swizzle, see ds_store_addr), one
+// 128-byte row of 64 query-row columns per key, 16-byte chunks XOR-swizzled like every staged
+// tile.  A 32-row block that is skipped stores zeros.  The wavefronts that form dQ read it back
+// with the transposing fragment reads.
+template <bool MASKED, bool DOCS, int NB, bool STORE_DS = false>
 __device__ __forceinline__ void dkdv_tile(uint32_t qsm, uint32_t gsm, uint32_t stat_lane, const TileLaneOffsets &lo,
                                           const bf16x8 (&kf)[NB][4], const bf16x8 (&vf)[NB][4],
                                           f32x16 (&dk)[NB][2], f32x16 (&dv)[NB][2], float c, int half,
                                           const int (&dbase)[NB], unsigned weff, int row_lim, int krel,
-                                          uint32_t ds_lane, const int (&jkey)[NB]) {
+                                          uint32_t ds_lane, const int (&jkey)[NB], uint32_t ds_out = 0) {
+    static_assert(!STORE_DS || NB == 1, "the dS store is written for one 32-key block per wavefront");
     // qsm / gsm: LDS byte addresses of the staged Q and dO tiles; stat_lane: address of this
     // lane's first lse2 value (rows 4*half..), -delta sits kTile floats further on.
     // DOCS (packed rows): ds_lane addresses the staged document starts of the same rows, jkey
@@ -110,7 +143,10 @@ __device__ __forceinline__ void dkdv_tile(uint32_t qsm, uint32_t gsm, uint32_t s
     // window, is skipped.
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) {
-        if (MASKED && ((32 * qb + 31 < krel) || (32 * qb > krel + 32 * NB - 1 + (int)weff - 1) || (32 * qb >= row_lim))) continue;
+        if (MASKED && ((32 * qb + 31 < krel) || (32 * qb > krel + 32 * NB - 1 + (int)weff - 1) || (32 * qb >= row_lim))) {
+            if constexpr (STORE_DS) ds_store_zero(ds_out, qb);
+            continue;
+        }
         f32x16 s[NB], dp[NB];
         // the dP accumulators start at -delta of their rows, so the MFMAs deliver dP - delta
 #pragma unroll
@@ -163,6 +199,7 @@ __device__ __forceinline__ void dkdv_tile(uint32_t qsm, uint32_t gsm, uint32_t s
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) {
                 const bf16x8 pf = cfrag(s[nb], u), dsf = cfrag(dp[nb], u);
+                if constexpr (STORE_DS) ds_store(ds_out, qb, u, dsf);
 #pragma unroll
                 for (int dblk = 0; dblk < 2; ++dblk) {
                     dv[nb][dblk] = mfma_bf16(agt[dblk], pf, dv[nb][dblk]);

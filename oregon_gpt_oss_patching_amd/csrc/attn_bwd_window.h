@@ -1,0 +1,415 @@
+// Single-pass backward for sliding-window layers (window <= 128): dQ, dK, dV and the dSinks
+// terms from ONE read of Q, dO, O, K, V, five GEMMs per (query tile, key tile) pair.  Stands in for
+// the reference's `_attn_bwd_precompute_D` + `_attn_bwd` (attention_kernel.py:102-217) on such
+// layers; results are bit-reproducible (no atomics, fixed summation orders).
+//
+// With a window of at most 128 a 64-row query tile t sees the three 64-key tiles t-2, t-1, t,
+// and a key tile is seen by the query tiles t, t+1, t+2.  A workgroup owns a chunk of
+// consecutive query tiles [t0, t1) of one KV head (all r query heads of the group) and walks
+// (query tile, head), heads inner.  Eight wavefronts:
+//   * six "owners", in three pairs; pair p holds, as MFMA B operands in registers, the K and V
+//     rows of the one live key tile kt with kt % 3 == p (32 keys per wavefront) and that tile's
+//     dK / dV accumulators.  Per iteration an owner does what the dK/dV kernel does for its keys
+//     (S = Q K^T, dP = dO V^T, P, dS, dV^T += dO^T P, dK^T += Q^T dS; see dkdv_tile) and leaves the
+//     bf16 dS block in LDS, key-major.  When the walk moves on to query tile t, key tile t-3 is
+//     complete: its pair writes dK / dV out and takes over key tile t.
+//   * two "helpers".  Helper hh owns rows 32*hh .. 32*hh+31 of every query tile: one iteration
+//     AHEAD of the owners it forms the row statistics lse*log2(e) and -rowsum(dO*O) of its rows
+//     (from O and dO rows it reads itself) and leaves them in LDS; one iteration BEHIND them it
+//     turns the dS tile into dQ^T = K^T dS^T over all 192 live keys (K fragments of the three live
+//     key tiles resident in its registers) and writes the finished dQ rows.  It also sums the
+//     dSinks terms exp(sink - lse) * (-delta) of its rows.
+// All 192 keys a query tile can see are in the workgroup at the same time, so dQ is complete
+// when the helper stores it.  dK / dV of the chunk's own key tiles [t0, t1) are complete once the
+// walk has gone two query tiles past the chunk (tiles t1, t1+1 are walked for their sake only);
+// the two key tiles before the chunk are walked for the sake of dQ only and their dK / dV are
+// dropped: the neighbouring chunk produces them.  That recomputation replaces any exchange of
+// partial sums between workgroups.
+//
+// One barrier per iteration hands over the staged Q / dO tile (asynchronous global->LDS copies,
+// three stages), the row statistics of the next tile and the dS tile of the previous one (double
+// buffered).  K / V rows of the next key tile travel through an LDS transit buffer one query
+// tile ahead of their use.
+#pragma once
+#include <type_traits>
+
+#include "attn_bwd.h"
+#include "attn_common.h"
+
+namespace gptoss {
+
+struct WinCfg {
+    static constexpr int NOWN = 6, NHELP = 2, NWAVES = NOWN + NHELP, NS = 3;
+    static constexpr int kMaxWindow = 128;
+    static constexpr int kMaxGroup = 64;                                   // query heads per KV head
+    static constexpr int kStageOff = 0;                                    // [NS][Q, dO][8 KB]
+    static constexpr int kStatOff = kStageOff + NS * 2 * kStageTileBytes;  // [NS][lse2, -delta][64] floats
+    static constexpr int kDsOff = kStatOff + NS * 2 * kTile * 4;           // [2][3 slabs of 64 keys][8 KB]
+    static constexpr int kDsBytes = 3 * kStageTileBytes;
+    static constexpr int kTransitOff = kDsOff + 2 * kDsBytes;              // [K, V][8 KB] of the next key tile
+    static constexpr int kOutOff = kTransitOff + 2 * kStageTileBytes;      // [NWAVES][32 x kLS] bf16 output stages
+    static constexpr int kSinkOff = kOutOff + NWAVES * 32 * kLS * 2;       // [NHELP][kMaxGroup] floats
+    static constexpr int kLdsBytes = kSinkOff + NHELP * kMaxGroup * 4;
+    static_assert(kDsOff % 128 == 0 && kTransitOff % 128 == 0, "swizzled tiles start on 128-byte boundaries");
+    static_assert(kLdsBytes <= 160 * 1024, "one workgroup per CU");
+};
+
+// (query tile, head within the group) of a position of the walk
+struct WinPos {
+    int t, h;
+    __device__ __forceinline__ void step(int r) { if (++h == r) { h = 0; ++t; } }
+};
+
+__global__ __launch_bounds__(WinCfg::NWAVES * 64, 1) void attn_bwd_window_kernel(const KArgs a) {
+    using C = WinCfg;
+    constexpr int NS = C::NS;
+    extern __shared__ __attribute__((aligned(1024))) char lds[];
+    char *const smem = lds + C::kStageOff;
+    float *const sstat = reinterpret_cast<float *>(lds + C::kStatOff);
+    char *const dsbuf = lds + C::kDsOff;
+    char *const transit = lds + C::kTransitOff;
+    float *const ssink = reinterpret_cast<float *>(lds + C::kSinkOff);
+
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int l32 = lane & 31, half = lane >> 5;
+    const bool owner = w < C::NOWN;
+
+    int bid = blockIdx.x;
+    const int g = bid % a.G; bid /= a.G;
+    const int b = bid % a.B; bid /= a.B;
+    const int chunk = bid;
+    const int n_chunks = gridDim.x / (a.G * a.B);
+    const int nT = (a.Sq + kTile - 1) / kTile;
+    const int t0 = chunk * a.chunk_tiles;                  // first query tile (and first own key tile)
+    const int t1 = min(t0 + a.chunk_tiles, nT);            // end of the chunk
+    const int t_end = min(t1 + 2, nT);                     // two more query tiles complete the chunk's dK / dV
+    const int n_it = (t_end - t0) * a.r;
+
+    const int kv_len = a.seqlens ? min(a.Skv, a.seqlens[b]) : a.Skv;
+    const int q_len = a.seqlens ? a.seqlens[b] : 0x7fffffff;
+    const int weff = a.window;
+
+    const TileLaneOffsets lo = make_tile_offsets(lane);
+    const uint32_t smem_base = lds_addr(smem), stat_base = lds_addr(sstat), ds_base = lds_addr(dsbuf);
+    const uint32_t transit_base = lds_addr(transit);
+    const bf16 *kbase = a.k + (int64_t)b * a.ks.b + (int64_t)g * a.ks.h;
+    const bf16 *vbase = a.v + (int64_t)b * a.vs.b + (int64_t)g * a.vs.h;
+    bf16 *const out_stage = reinterpret_cast<bf16 *>(lds + C::kOutOff) + w * 32 * kLS;
+
+    // key tile that pair / slot p holds while the walk is at query tile t: the one of t-2, t-1, t
+    // that is congruent to p modulo 3
+    auto tile_of_slot = [](int p, int t) { return t - ((t - p) % 3 + 3) % 3; };
+
+    // ---- prologue: the three key tiles live at the first query tile --------------------------
+    // Their K rows go through LDS (slab p of the first dS buffer) so that the helpers can pick
+    // them up as transposed fragments; rows outside the tensor repeat a valid row (finite values
+    // that only ever meet dS = 0).
+    for (int slot = w; slot < 24; slot += C::NWAVES) {
+        const int p = slot >> 3, r8 = slot & 7;
+        const int kt = tile_of_slot(p, t0);
+        const int rr = 8 * r8 + (lane >> 3);
+        const int cc = (lane & 7) ^ swz(rr);
+        const int row = min(max(kt * kTile + rr, 0), a.Skv - 1);
+        __builtin_amdgcn_global_load_lds((glb_void_t *)(kbase + (int64_t)row * a.ks.s + cc * 8),
+                                         (lds_void_t *)(dsbuf + p * kStageTileBytes + r8 * 8 * kRowBytes), 16, 0, 0);
+    }
+
+    if (!owner) {
+        // =================================== helper wavefronts ===================================
+        const int hh = w - C::NOWN;
+        const int srow = 32 * hh + (lane >> 1), hr = lane & 1;     // statistics: two lanes per row, 32 columns each
+        if (lane < a.r) ssink[hh * C::kMaxGroup + lane] = 0.0f;
+        const float *sinks = a.sinks;
+
+        // O and dO half rows + lse of this lane's row of walk position `pos`
+        u32x4 pre_o[4], pre_g[4];
+        float pre_lse = 0.0f;
+        auto prefetch = [&](const WinPos &pos) {
+            const int head = g * a.r + pos.h;
+            const int row = min(pos.t * kTile + srow, a.Sq - 1);
+            const bf16 *orow = a.o + (int64_t)b * a.os.b + (int64_t)head * a.os.h + (int64_t)row * a.os.s + 32 * hr;
+            const bf16 *grow = a.d_o + (int64_t)b * a.dos.b + (int64_t)head * a.dos.h + (int64_t)row * a.dos.s + 32 * hr;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                pre_o[j] = *reinterpret_cast<const u32x4 *>(orow + 8 * j);
+                pre_g[j] = *reinterpret_cast<const u32x4 *>(grow + 8 * j);
+            }
+            pre_lse = a.lse[((int64_t)b * a.H + head) * a.Sq + row];
+        };
+        // row statistics of the prefetched rows into stage `stage`; dSinks terms of own rows
+        auto statistics = [&](const WinPos &pos, int stage) {
+            float acc = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const bf16x8 of = as_bf16x8(pre_o[j]), gf = as_bf16x8(pre_g[j]);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) acc = fmaf((float)of[e], (float)gf[e], acc);
+            }
+            acc += __shfl_xor(acc, 1);
+            const float lse2 = pre_lse * kLog2e;
+            if (hr == 0) {
+                sstat[(stage * 2 + 0) * kTile + srow] = lse2;
+                sstat[(stage * 2 + 1) * kTile + srow] = -acc;
+            }
+            if (a.dsinks && pos.t < t1) {                       // rows of the chunk itself, each counted once
+                const float sink2 = (sinks ? sinks[g * a.r + pos.h] : 0.0f) * kLog2e;
+                float term = (hr == 0 && pos.t * kTile + srow < a.Sq) ? fast_exp2(sink2 - lse2) * -acc : 0.0f;
+#pragma unroll
+                for (int off = 32; off > 0; off >>= 1) term += __shfl_xor(term, off);
+                if (lane == 0) ssink[hh * C::kMaxGroup + pos.h] += term;
+            }
+        };
+
+        WinPos p_stat{t0, 0}, p_pre{t0, 0}, p_prev{t0, 0};
+        prefetch(p_pre);
+        p_pre.step(a.r);
+        wait_vmcnt<0>();
+        __syncthreads();                                       // the K slabs are in LDS
+        // K^T fragments (A operands: lane = column, slots = keys) of the three live key tiles
+        bf16x8 kfr[3][4][2];
+#pragma unroll
+        for (int p = 0; p < 3; ++p)
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+                for (int db = 0; db < 2; ++db) kfr[p][kk][db] = ofrag_tr(ds_base + p * kStageTileBytes, lo, kk >> 1, kk & 1, db);
+        statistics(p_stat, 0);                                 // statistics of the first tile
+        p_stat.step(a.r);
+        if (n_it > 1) { prefetch(p_pre); p_pre.step(a.r); }
+
+        // dQ rows 32*hh.. of the tile at `pos` from the dS tile at LDS address ds_tile
+        auto helper_dq = [&](uint32_t ds_tile, const WinPos &pos) {
+            f32x16 acc[2];
+#pragma unroll
+            for (int db = 0; db < 2; ++db)
+#pragma unroll
+                for (int i = 0; i < 16; ++i) acc[db][i] = 0.0f;
+#pragma unroll
+            for (int p = 0; p < 3; ++p)
+#pragma unroll
+                for (int kk = 0; kk < 4; ++kk) {
+                    const bf16x8 ads = ofrag_tr(ds_tile + p * kStageTileBytes, lo, kk >> 1, kk & 1, hh);
+#pragma unroll
+                    for (int db = 0; db < 2; ++db) acc[db] = mfma_bf16(kfr[p][kk][db], ads, acc[db]);
+                }
+            const int r0 = pos.t * kTile + 32 * hh;
+            const int head = g * a.r + pos.h;
+            bf16 *row0 = a.dq + (int64_t)b * a.dqs.b + (int64_t)head * a.dqs.h + (int64_t)r0 * a.dqs.s;
+            store_rows32(out_stage, acc, a.scale, row0, a.dqs.s, a.Sq - r0, lane);
+            __builtin_amdgcn_wave_barrier();
+        };
+        auto reload = [&](auto slot_tag) {
+            constexpr int P = decltype(slot_tag)::value;
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk)
+#pragma unroll
+                for (int db = 0; db < 2; ++db) kfr[P][kk][db] = ofrag_tr(transit_base, lo, kk >> 1, kk & 1, db);
+        };
+
+        WinPos cur{t0, 0};
+        for (int it = 0; it < n_it; ++it) {
+            __syncthreads();
+            if (it > 0 && p_prev.t < t1) helper_dq(ds_base + ((it - 1) & 1) * C::kDsBytes, p_prev);
+            if (cur.h == 0 && cur.t > t0 && cur.t < t1) {
+                // key tile cur.t has arrived in the transit buffer; it replaces tile cur.t - 3
+                const int slot = cur.t % 3;
+                if (slot == 0) reload(std::integral_constant<int, 0>{});
+                else if (slot == 1) reload(std::integral_constant<int, 1>{});
+                else reload(std::integral_constant<int, 2>{});
+            }
+            if (it + 1 < n_it) {
+                statistics(p_stat, (it + 1) % NS);
+                p_stat.step(a.r);
+            }
+            if (it + 2 < n_it) {
+                prefetch(p_pre);
+                p_pre.step(a.r);
+            }
+            p_prev = cur;
+            cur.step(a.r);
+        }
+        __syncthreads();                                       // the last dS tile is complete
+        if (p_prev.t < t1) helper_dq(ds_base + ((n_it - 1) & 1) * C::kDsBytes, p_prev);
+        if (a.dsinks && lane < a.r)
+            a.dsink_partial[((((int64_t)b * n_chunks + chunk) * a.G + g) * a.r + lane) * C::NHELP + hh] = ssink[hh * C::kMaxGroup + lane];
+        return;
+    }
+
+    // ===================================== owner wavefronts =====================================
+    const int pair = w >> 1, sub = w & 1;
+    int my_kt = tile_of_slot(pair, t0);                        // key tile held (negative: none yet)
+    bf16x8 kf[1][4], vf[1][4];
+    f32x16 dk[1][2], dv[1][2];
+    auto clear_acc = [&]() {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) { dk[0][0][i] = dk[0][1][i] = 0.0f; dv[0][0][i] = dv[0][1][i] = 0.0f; }
+    };
+    {
+        const int j = my_kt * kTile + 32 * sub + l32;
+        const bool ok = my_kt >= 0 && j < a.Skv;
+        const bf16 *krow = kbase + (int64_t)(ok ? j : 0) * a.ks.s;
+        const bf16 *vrow = vbase + (int64_t)(ok ? j : 0) * a.vs.s;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            u32x4 zk = {0u, 0u, 0u, 0u}, zv = {0u, 0u, 0u, 0u};
+            if (ok) {
+                zk = *reinterpret_cast<const u32x4 *>(krow + 16 * ks + 8 * half);
+                zv = *reinterpret_cast<const u32x4 *>(vrow + 16 * ks + 8 * half);
+            }
+            kf[0][ks] = as_bf16x8(zk);
+            vf[0][ks] = as_bf16x8(zv);
+        }
+        clear_acc();
+    }
+    // dK / dV of the key tile held, if it is one of the chunk's own
+    auto flush = [&]() {
+        if (my_kt < t0 || my_kt >= t1) return;
+        const int r0 = my_kt * kTile + 32 * sub;
+        const int nvalid = a.Skv - r0;
+        store_rows32(out_stage, dk[0], a.scale, a.dk + (int64_t)b * a.dks.b + (int64_t)g * a.dks.h + (int64_t)r0 * a.dks.s,
+                     a.dks.s, nvalid, lane);
+        __builtin_amdgcn_wave_barrier();
+        store_rows32(out_stage, dv[0], 1.0f, a.dv + (int64_t)b * a.dvs.b + (int64_t)g * a.dvs.h + (int64_t)r0 * a.dvs.s,
+                     a.dvs.s, nvalid, lane);
+        __builtin_amdgcn_wave_barrier();
+    };
+
+    const float c = a.scale_log2;
+    int dead[1] = {0};
+    const uint32_t ds_out0 = ds_store_addr(ds_base + pair * kStageTileBytes, 32 * sub + l32, half);
+
+    // ---- copies: wavefront 0 the Q tile, wavefront 1 the dO tile of each walk position (eight
+    // 16-byte-per-lane instructions), wavefront 2 the K and V rows of the next key tile ----
+    const int64_t lstride = (w == 0) ? a.qs.s : a.dos.s;
+    const int64_t ld_hstride = (w == 0) ? a.qs.h : a.dos.h;
+    uint32_t ld_off[2];
+    {
+        const int lr = lane >> 3;
+        ld_off[0] = (uint32_t)(lr * (int)lstride + (((lane & 7) ^ swz(lr)) * 8));
+        ld_off[1] = (uint32_t)(lr * (int)lstride + (((lane & 7) ^ swz(lr + 8)) * 8));
+    }
+    int iss_h = 0, iss_i0 = t0 * kTile;
+    const bf16 *ld_tile = (w == 0)
+        ? a.q + (int64_t)b * a.qs.b + (int64_t)(g * a.r) * a.qs.h + (int64_t)iss_i0 * a.qs.s
+        : a.d_o + (int64_t)b * a.dos.b + (int64_t)(g * a.r) * a.dos.h + (int64_t)iss_i0 * a.dos.s;
+    auto issue = [&](int it) {
+        const int stage = it % NS;
+        if (w < 2) {
+            char *dst = smem + (stage * 2 + w) * kStageTileBytes;
+            if (iss_i0 + kTile <= a.Sq) {
+#pragma unroll
+                for (int k = 0; k < 8; ++k)
+                    __builtin_amdgcn_global_load_lds((glb_void_t *)(ld_tile + (int64_t)(8 * k) * lstride + ld_off[k & 1]),
+                                                     (lds_void_t *)(dst + 8 * k * kRowBytes), 16, 0, 0);
+            } else {
+                // the tile sticks out of the tensor: rows past the end re-read the last valid one
+                // (rare: a rolled loop keeps its address arithmetic out of the registers of the main loop)
+#pragma unroll 1
+                for (int k = 0; k < 8; ++k) {
+                    const int rr = 8 * k + (lane >> 3);
+                    const int cc = (lane & 7) ^ swz(rr);
+                    const int over = max(0, iss_i0 + rr - (a.Sq - 1));
+                    __builtin_amdgcn_global_load_lds((glb_void_t *)(ld_tile + (int64_t)(rr - over) * lstride + cc * 8),
+                                                     (lds_void_t *)(dst + 8 * k * kRowBytes), 16, 0, 0);
+                }
+            }
+        }
+        ++iss_h;
+        ld_tile += ld_hstride;
+        if (iss_h == a.r) {
+            iss_h = 0;
+            iss_i0 += kTile;
+            ld_tile += (int64_t)kTile * lstride - (int64_t)a.r * ld_hstride;
+        }
+    };
+    auto issue_transit = [&](int kt) {
+#pragma unroll 1
+        for (int k = 0; k < 8; ++k) {
+            const int rr = 8 * k + (lane >> 3);
+            const int cc = (lane & 7) ^ swz(rr);
+            const int row = min(kt * kTile + rr, a.Skv - 1);
+            __builtin_amdgcn_global_load_lds((glb_void_t *)(kbase + (int64_t)row * a.ks.s + cc * 8),
+                                             (lds_void_t *)(transit + 8 * k * kRowBytes), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((glb_void_t *)(vbase + (int64_t)row * a.vs.s + cc * 8),
+                                             (lds_void_t *)(transit + kStageTileBytes + 8 * k * kRowBytes), 16, 0, 0);
+        }
+    };
+
+    wait_vmcnt<0>();
+    __syncthreads();                                           // prologue barrier (the helpers read the K slabs now)
+    issue(0);
+    if (n_it > 1) issue(1);
+
+    WinPos cur{t0, 0};
+    auto iterate = [&](int it, auto stage_tag) {
+        constexpr int STAGE = decltype(stage_tag)::value;
+        if (w < 2) { if (it + 1 >= n_it) wait_vmcnt<0>(); else wait_vmcnt<8>(); }
+        else if (w == 2 && cur.h == 0) wait_vmcnt<0>();        // the transit copy of the key tile that starts now
+        __syncthreads();
+        if (it + 2 < n_it) issue(it + 2);
+        if (w == 2 && cur.h == 1 && cur.t + 1 < t1) issue_transit(cur.t + 1);
+
+        if (cur.h == 0 && cur.t > t0 && pair == cur.t % 3) {
+            // this pair's key tile (cur.t - 3) is complete; take over key tile cur.t from the transit buffer
+            flush();
+            my_kt = cur.t < t1 ? cur.t : -1;
+            if (my_kt >= 0) {
+#pragma unroll
+                for (int ks = 0; ks < 4; ++ks) {
+                    kf[0][ks] = ofrag_nat(transit_base, lo, sub, ks);
+                    vf[0][ks] = ofrag_nat(transit_base + kStageTileBytes, lo, sub, ks);
+                }
+            }
+            clear_acc();
+        }
+
+        const int i0 = cur.t * kTile;
+        const uint32_t ds_out = ds_out0 + (it & 1) * C::kDsBytes;
+        const int wj0 = my_kt * kTile + 32 * sub;              // first key of the wavefront
+        const int pos0 = i0;
+        const int pos1 = min(min(a.Sq, i0 + kTile) - 1, q_len - 1);
+        const int wj1 = min(wj0 + 32, kv_len) - 1;
+        const bool skip = my_kt < 0 || wj1 < wj0 || pos1 < wj0 || pos0 > wj1 + weff - 1 || pos1 < pos0;
+        if (skip) {
+            ds_store_zero(ds_out, 0);
+            ds_store_zero(ds_out, 1);
+        } else {
+            const uint32_t qsm = smem_base + STAGE * (2 * kStageTileBytes), gsm = qsm + kStageTileBytes;
+            const uint32_t stat_lane = stat_base + STAGE * (2 * kTile * 4) + half * 16;
+            const bool interior = (wj0 + 31 <= pos0) && (wj0 > pos1 - weff) && (wj0 + 32 <= kv_len) && (i0 + kTile - 1 <= pos1);
+            int jkey[1] = {wj0 + l32};
+            if (interior) {
+                dkdv_tile<false, false, 1, true>(qsm, gsm, stat_lane, lo, kf, vf, dk, dv, c, half, dead, 0u, 0, 0, 0u, jkey, ds_out);
+            } else {
+                int dbase[1];
+                dbase[0] = (wj0 + l32 < kv_len) ? pos0 - (wj0 + l32) : -0x40000000;
+                const int row_lim = min(kTile, min(a.Sq, q_len) - i0);
+                dkdv_tile<true, false, 1, true>(qsm, gsm, stat_lane, lo, kf, vf, dk, dv, c, half, dbase, (unsigned)weff, row_lim,
+                                                wj0 - pos0, 0u, jkey, ds_out);
+            }
+        }
+        cur.step(a.r);
+    };
+
+    for (int it = 0; it < n_it; it += NS) {
+        iterate(it, std::integral_constant<int, 0>{});
+        if (it + 1 < n_it) iterate(it + 1, std::integral_constant<int, 1>{});
+        if (it + 2 < n_it) iterate(it + 2, std::integral_constant<int, 2>{});
+    }
+    __syncthreads();                                           // hands the last dS tile over
+    flush();
+}
+
+// ---------------------------------------------------------------------------------
+// dsinks[h] = sum of the per-(batch, chunk, helper) partial sums the window kernel left, in a
+// fixed order.  One thread per query head.
+__global__ __launch_bounds__(64) void attn_bwd_window_dsinks_kernel(const KArgs a, int n_chunks) {
+    const int h = blockIdx.x * 64 + threadIdx.x;
+    if (h >= a.H) return;
+    float acc = 0.0f;
+    for (int bc = 0; bc < a.B * n_chunks; ++bc)
+        for (int e = 0; e < WinCfg::NHELP; ++e) acc += a.dsink_partial[((int64_t)bc * a.H + h) * WinCfg::NHELP + e];
+    a.dsinks[h] = acc;
+}
+
+}  // namespace gptoss

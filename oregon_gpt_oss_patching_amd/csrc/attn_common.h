@@ -53,6 +53,8 @@ struct KArgs {
     float scale_log2;    // scale * log2(e)
     int dkdv_parts;      // dK/dV kernel: workgroups that share one key block, each taking a slice of its query tiles
     float *dkdv_partial; // dkdv_parts > 1: fp32 partial sums, [part][dK, dV][B][G][Skv][64]
+    int chunk_tiles;     // single-pass window backward: 64-row query tiles per workgroup
+    float *dsink_partial; // single-pass window backward: dSinks partial sums, [B][chunk][H][2]
 };
 
 __device__ __forceinline__ int crow(int i, int half) { return 8 * (i >> 2) + 4 * half + (i & 3); }

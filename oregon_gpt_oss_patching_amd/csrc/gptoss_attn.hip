@@ -7,6 +7,7 @@
 
 #include "../../include/gptoss_attn.h"
 #include "attn_bwd.h"
+#include "attn_bwd_window.h"
 #include "attn_common.h"
 #include "attn_f32.h"
 #include "attn_fwd.h"
@@ -54,6 +55,8 @@ KArgs make_args(const gptoss_attn_params *p) {
     a.scale = p->scale;
     a.scale_log2 = p->scale * kLog2e;
     a.dkdv_parts = 1;
+    a.chunk_tiles = 0;
+    a.dsink_partial = nullptr;
     return a;
 }
 
@@ -93,11 +96,75 @@ int64_t f32_grid(int64_t waves) { return (waves + 3) / 4; }
 // thread left in the runtime's sticky state is neither reported here nor cleared.  A grid beyond the
 // x-dimension limit is refused on the host.
 template <typename Kernel>
-int launch(Kernel kernel, int64_t workgroups, int threads, hipStream_t st, const KArgs &a) {
+int launch(Kernel kernel, int64_t workgroups, int threads, hipStream_t st, const KArgs &a, size_t dynamic_lds = 0) {
     if (workgroups <= 0 || workgroups > 0x7fffffff) return GPTOSS_ATTN_ERR_SHAPE;
     void *args[] = {const_cast<KArgs *>(&a)};
     const hipError_t e = hipLaunchKernel(reinterpret_cast<const void *>(kernel), dim3((unsigned)workgroups), dim3((unsigned)threads),
-                                         args, 0, st);
+                                         args, dynamic_lds, st);
+    return e == hipSuccess ? GPTOSS_ATTN_OK : static_cast<int>(e);
+}
+
+// ---- single-pass backward of sliding-window layers (attn_bwd_window.h) ------------------------
+// Taken for bf16 self-attention (Sq == Skv, no offset, no packed rows) with a window of at most
+// 128 and 2..64 query heads per KV head; everything else keeps the dK/dV + dQ kernel pair.
+bool window_single_pass(const gptoss_attn_params *p) {
+    const int r = p->G > 0 ? p->H / p->G : 0;
+    return p->dtype == GPTOSS_ATTN_BF16 && p->window > 0 && p->window <= WinCfg::kMaxWindow && !p->doc_start &&
+           p->q_offset == 0 && p->Sq == p->Skv && r >= 2 && r <= WinCfg::kMaxGroup;
+}
+
+constexpr int kMaxDevices = 64;
+
+// Compute units of the current device (looked up once per device).
+int compute_units() {
+    static std::atomic<int> cus[kMaxDevices];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+    int n = cus[dev].load(std::memory_order_acquire);
+    if (n <= 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cus[dev].store(n, std::memory_order_release);
+    }
+    return n;
+}
+
+// Query tiles per workgroup: about one workgroup per compute unit, between 2 and 16 tiles (each
+// workgroup walks two tiles beyond its own, so short chunks repeat more work).
+int window_chunk_tiles(const gptoss_attn_params *p, int cus) {
+    const int64_t tiles = (int64_t)((p->Sq + kTile - 1) / kTile) * p->G * p->B;
+    int64_t c = tiles / (cus > 0 ? cus : 256);
+    return (int)(c < 2 ? 2 : (c > 16 ? 16 : c));
+}
+
+// A kernel that uses more than 64 KB of LDS has to be told so once per device.
+int window_lds_attribute() {
+    static std::atomic<bool> done[kMaxDevices];
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return static_cast<int>(e);
+    const bool tracked = dev >= 0 && dev < kMaxDevices;
+    if (!tracked || !done[dev].load(std::memory_order_acquire)) {
+        e = hipFuncSetAttribute(reinterpret_cast<const void *>(attn_bwd_window_kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                WinCfg::kLdsBytes);
+        if (e != hipSuccess) return static_cast<int>(e);
+        if (tracked) done[dev].store(true, std::memory_order_release);
+    }
+    return GPTOSS_ATTN_OK;
+}
+
+int launch_window_bwd(const gptoss_attn_params *p, hipStream_t st) {
+    int rc = window_lds_attribute();
+    if (rc) return rc;
+    KArgs a = make_args(p);
+    a.chunk_tiles = window_chunk_tiles(p, compute_units());
+    a.dsink_partial = p->delta;                       // the row-statistics part of the scratch is free in this path
+    const int n_tiles = (a.Sq + kTile - 1) / kTile;
+    const int n_chunks = (n_tiles + a.chunk_tiles - 1) / a.chunk_tiles;
+    rc = launch(attn_bwd_window_kernel, (int64_t)a.G * a.B * n_chunks, 64 * WinCfg::NWAVES, st, a, WinCfg::kLdsBytes);
+    if (rc || !a.dsinks) return rc;
+    void *args[] = {&a, const_cast<int *>(&n_chunks)};
+    const hipError_t e = hipLaunchKernel(reinterpret_cast<const void *>(attn_bwd_window_dsinks_kernel), dim3((unsigned)((a.H + 63) / 64)),
+                                         dim3(64), args, 0, st);
     return e == hipSuccess ? GPTOSS_ATTN_OK : static_cast<int>(e);
 }
 
@@ -256,6 +323,7 @@ static int bwd_all(const gptoss_attn_params *p, void *stream, bool whole_blocks)
         if (rc) return rc;
         return gptoss_attn_bwd_dq(p, stream);
     }
+    if (window_single_pass(p)) return launch_window_bwd(p, static_cast<hipStream_t>(stream));
     rc = launch_dq(p, stream, 1);
     if (rc) return rc;
     if (p->dsinks) {
@@ -274,7 +342,6 @@ int gptoss_attn_bwd(const gptoss_attn_params *p, void *stream) { return bwd_all(
 // at its own address, looked up once per device.
 namespace {
 constexpr size_t kStaticScratchBytes = GPTOSS_ATTN_STATIC_SCRATCH_BYTES;
-constexpr int kMaxDevices = 64;
 }
 static __device__ __align__(256) float scratch[kStaticScratchBytes / sizeof(float)];
 static std::atomic<float *> scratch_ptr[kMaxDevices];     // device address of `scratch`, per device; NULL = not looked up yet

@@ -380,32 +380,48 @@ def test_null_sinks_is_zero_logit(A):
     assert ds is None and torch.isfinite(dq).all()
 
 
-def test_deterministic_bitwise(A):
+@pytest.mark.parametrize("w", [None, 128, 40])
+def test_deterministic_bitwise(A, w):
+    """Two runs give the same bits, on every path: the dK/dV + dQ kernel pair (full causal) and the
+    single-pass backward of sliding-window layers (no atomics anywhere)."""
     inp = E.make_inputs(61, 1, 64, 8, 1024, 64, torch.bfloat16)
-    a = run_hip(A, *inp, None)
-    b = run_hip(A, *inp, None)
+    a = run_hip(A, *inp, w)
+    b = run_hip(A, *inp, w)
     for x, y in zip(a, b):
         assert torch.equal(x, y)
 
 
 @pytest.mark.parametrize("b,h,g,s,w,lens,docs", [
     (1, 64, 8, 1024, None, None, None), (1, 8, 2, 333, 32, None, None), (2, 8, 2, 200, None, [150, 77], None),
-    (1, 8, 2, 300, 128, None, [100, 120, 80]), (1, 6, 3, 130, 50, None, None),
+    (1, 8, 2, 300, 128, None, [100, 120, 80]), (1, 6, 3, 130, 50, None, None), (1, 8, 2, 300, 200, None, None),
+    (2, 16, 2, 700, 128, [700, 333], None),
 ])
 def test_combined_backward_equals_separate_steps(A, b, h, g, s, w, lens, docs):
-    """gptoss_attn_bwd (dQ kernel computes delta and lse*log2e itself, then dSinks, dK/dV) against
-    preprocess + dK/dV + dQ called one after the other: the same bits in every output."""
+    """gptoss_attn_bwd against preprocess + dK/dV + dQ called one after the other.  Where
+    gptoss_attn_bwd runs the same kernels (its dQ kernel computes delta and lse*log2e itself, then
+    dSinks, dK/dV) every output has the same bits.  Sliding-window layers with a window of at most
+    128 and no packed rows take the single-pass kernel instead, which sums dQ over keys and dK/dV
+    over rows in another order: there the two agree to the last bf16 bit or two."""
     q, k, v, sinks, d_out = (t.to(DEV) for t in E.make_inputs(900 + s, b, h, g, s, 64, torch.bfloat16))
     doc_start = None
     if docs is not None:
         starts = torch.tensor([0] + list(np.cumsum(docs)[:-1]), dtype=torch.int32)
         doc_start = torch.repeat_interleave(starts, torch.tensor(docs)).view(1, s).to(DEV)
+    if lens is not None:
+        d_out = mask_dout(d_out.cpu(), lens).to(DEV)
     o, lse = A.attention_forward(q, k, v, sinks, SCALE, w, 0, lens, doc_start)
     one = A.attention_backward(q, k, v, sinks, o, lse, d_out, SCALE, w, 0, lens, doc_start=doc_start)
     three = A.attention_backward(q, k, v, sinks, o, lse, d_out, SCALE, w, 0, lens, doc_start=doc_start, split=True)
     torch.cuda.synchronize()
-    for x, y in zip(one, three):
-        assert torch.equal(x, y)
+    single_pass = w is not None and w <= 128 and docs is None and h // g >= 2
+    for name, x, y in zip(("dq", "dk", "dv", "dsinks"), one, three):
+        if not single_pass:
+            assert torch.equal(x, y), name
+            continue
+        x, y = x.float(), y.float()
+        assert rel_l2(x, y) <= 1e-4, (name, rel_l2(x, y))
+        if name != "dsinks":
+            assert bool(((x - y).abs() <= 2.0 ** -7 * torch.maximum(x.abs(), y.abs()) + 1e-6).all()), name
 
 
 def test_window_ge_seq_equals_full(A):
