@@ -41,15 +41,15 @@ namespace gptoss {
 struct WinCfg {
     static constexpr int NOWN = 6, NHELP = 2, NWAVES = NOWN + NHELP, NS = 3;
     static constexpr int kMaxWindow = 128;
-    static constexpr int kMaxGroup = 64;                                   // query heads per KV head
+    static constexpr int kMaxGroup = 16;                                   // query heads per KV head
     static constexpr int kStageOff = 0;                                    // [NS][Q, dO][8 KB]
     static constexpr int kStatOff = kStageOff + NS * 2 * kStageTileBytes;  // [NS][lse2, -delta][64] floats
     static constexpr int kDsOff = kStatOff + NS * 2 * kTile * 4;           // [2][3 slabs of 64 keys][8 KB]
     static constexpr int kDsBytes = 3 * kStageTileBytes;
     static constexpr int kTransitOff = kDsOff + 2 * kDsBytes;              // [K, V][8 KB] of the next key tile
     static constexpr int kOutOff = kTransitOff + 2 * kStageTileBytes;      // [NWAVES][32 x kLS] bf16 output stages
-    static constexpr int kSinkOff = kOutOff + NWAVES * 32 * kLS * 2;       // [NHELP][kMaxGroup] floats
-    static constexpr int kLdsBytes = kSinkOff + NHELP * kMaxGroup * 4;
+    static constexpr int kSinkOff = kOutOff + NWAVES * 32 * kLS * 2;       // [NHELP][kMaxGroup][64 lanes] floats
+    static constexpr int kLdsBytes = kSinkOff + NHELP * kMaxGroup * 64 * 4;
     static_assert(kDsOff % 128 == 0 && kTransitOff % 128 == 0, "swizzled tiles start on 128-byte boundaries");
     static_assert(kLdsBytes <= 160 * 1024, "one workgroup per CU");
 };
@@ -118,33 +118,53 @@ __global__ __launch_bounds__(WinCfg::NWAVES * 64, 1) void attn_bwd_window_kernel
         // =================================== helper wavefronts ===================================
         const int hh = w - C::NOWN;
         const int srow = 32 * hh + (lane >> 1), hr = lane & 1;     // statistics: two lanes per row, 32 columns each
-        if (lane < a.r) ssink[hh * C::kMaxGroup + lane] = 0.0f;
+        // dSinks terms are summed per lane (own LDS slot per head, no cross-lane traffic in the loop)
+        float *const my_sink = ssink + (hh * C::kMaxGroup) * 64 + lane;
+        for (int h = 0; h < a.r; ++h) my_sink[h * 64] = 0.0f;
         const float *sinks = a.sinks;
 
-        // O and dO half rows + lse of this lane's row of walk position `pos`
+        // O and dO half rows + lse of this lane's row of walk position `pos`.  The row pointers
+        // follow the walk (heads inner, then the next query tile); the last tile's rows past the
+        // end of the tensor re-read the last valid row.
         u32x4 pre_o[4], pre_g[4];
         float pre_lse = 0.0f;
-        auto prefetch = [&](const WinPos &pos) {
-            const int head = g * a.r + pos.h;
-            const int row = min(pos.t * kTile + srow, a.Sq - 1);
-            const bf16 *orow = a.o + (int64_t)b * a.os.b + (int64_t)head * a.os.h + (int64_t)row * a.os.s + 32 * hr;
-            const bf16 *grow = a.d_o + (int64_t)b * a.dos.b + (int64_t)head * a.dos.h + (int64_t)row * a.dos.s + 32 * hr;
+        const int64_t stat_row0 = min(t0 * kTile + srow, a.Sq - 1);
+        const bf16 *orow = a.o + (int64_t)b * a.os.b + (int64_t)(g * a.r) * a.os.h + stat_row0 * a.os.s + 32 * hr;
+        const bf16 *grow = a.d_o + (int64_t)b * a.dos.b + (int64_t)(g * a.r) * a.dos.h + stat_row0 * a.dos.s + 32 * hr;
+        const float *lrow = a.lse + ((int64_t)b * a.H + (int64_t)g * a.r) * a.Sq + stat_row0;
+        auto prefetch = [&](WinPos &pos) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 pre_o[j] = *reinterpret_cast<const u32x4 *>(orow + 8 * j);
                 pre_g[j] = *reinterpret_cast<const u32x4 *>(grow + 8 * j);
             }
-            pre_lse = a.lse[((int64_t)b * a.H + head) * a.Sq + row];
+            pre_lse = *lrow;
+            orow += a.os.h;
+            grow += a.dos.h;
+            lrow += a.Sq;
+            if (++pos.h == a.r) {
+                pos.h = 0;
+                ++pos.t;
+                // rows of the next tile (clamped at the end of the tensor)
+                const int64_t adv = min(pos.t * kTile + srow, a.Sq - 1) - min((pos.t - 1) * kTile + srow, a.Sq - 1);
+                orow += adv * a.os.s - (int64_t)a.r * a.os.h;
+                grow += adv * a.dos.s - (int64_t)a.r * a.dos.h;
+                lrow += adv - (int64_t)a.r * a.Sq;
+            }
         };
         // row statistics of the prefetched rows into stage `stage`; dSinks terms of own rows
         auto statistics = [&](const WinPos &pos, int stage) {
+            typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
             float acc = 0.0f;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const bf16x8 of = as_bf16x8(pre_o[j]), gf = as_bf16x8(pre_g[j]);
+            for (int j = 0; j < 4; ++j)
 #pragma unroll
-                for (int e = 0; e < 8; ++e) acc = fmaf((float)of[e], (float)gf[e], acc);
-            }
+                for (int e = 0; e < 4; ++e) {
+                    union { uint32_t u; bf16x2 v; } x, y;
+                    x.u = pre_o[j][e];
+                    y.u = pre_g[j][e];
+                    acc = __builtin_amdgcn_fdot2_f32_bf16(x.v, y.v, acc, false);
+                }
             acc += __shfl_xor(acc, 1);
             const float lse2 = pre_lse * kLog2e;
             if (hr == 0) {
@@ -153,16 +173,13 @@ __global__ __launch_bounds__(WinCfg::NWAVES * 64, 1) void attn_bwd_window_kernel
             }
             if (a.dsinks && pos.t < t1) {                       // rows of the chunk itself, each counted once
                 const float sink2 = (sinks ? sinks[g * a.r + pos.h] : 0.0f) * kLog2e;
-                float term = (hr == 0 && pos.t * kTile + srow < a.Sq) ? fast_exp2(sink2 - lse2) * -acc : 0.0f;
-#pragma unroll
-                for (int off = 32; off > 0; off >>= 1) term += __shfl_xor(term, off);
-                if (lane == 0) ssink[hh * C::kMaxGroup + pos.h] += term;
+                const float term = (hr == 0 && pos.t * kTile + srow < a.Sq) ? fast_exp2(sink2 - lse2) * -acc : 0.0f;
+                my_sink[pos.h * 64] += term;
             }
         };
 
         WinPos p_stat{t0, 0}, p_pre{t0, 0}, p_prev{t0, 0};
         prefetch(p_pre);
-        p_pre.step(a.r);
         wait_vmcnt<0>();
         __syncthreads();                                       // the K slabs are in LDS
         // K^T fragments (A operands: lane = column, slots = keys) of the three live key tiles
@@ -175,7 +192,7 @@ __global__ __launch_bounds__(WinCfg::NWAVES * 64, 1) void attn_bwd_window_kernel
                 for (int db = 0; db < 2; ++db) kfr[p][kk][db] = ofrag_tr(ds_base + p * kStageTileBytes, lo, kk >> 1, kk & 1, db);
         statistics(p_stat, 0);                                 // statistics of the first tile
         p_stat.step(a.r);
-        if (n_it > 1) { prefetch(p_pre); p_pre.step(a.r); }
+        if (n_it > 1) prefetch(p_pre);
 
         // dQ rows 32*hh.. of the tile at `pos` from the dS tile at LDS address ds_tile
         auto helper_dq = [&](uint32_t ds_tile, const WinPos &pos) {
@@ -221,17 +238,20 @@ __global__ __launch_bounds__(WinCfg::NWAVES * 64, 1) void attn_bwd_window_kernel
                 statistics(p_stat, (it + 1) % NS);
                 p_stat.step(a.r);
             }
-            if (it + 2 < n_it) {
-                prefetch(p_pre);
-                p_pre.step(a.r);
-            }
+            if (it + 2 < n_it) prefetch(p_pre);
             p_prev = cur;
             cur.step(a.r);
         }
         __syncthreads();                                       // the last dS tile is complete
         if (p_prev.t < t1) helper_dq(ds_base + ((n_it - 1) & 1) * C::kDsBytes, p_prev);
-        if (a.dsinks && lane < a.r)
-            a.dsink_partial[((((int64_t)b * n_chunks + chunk) * a.G + g) * a.r + lane) * C::NHELP + hh] = ssink[hh * C::kMaxGroup + lane];
+        if (a.dsinks) {
+            for (int h = 0; h < a.r; ++h) {
+                float v = my_sink[h * 64];
+#pragma unroll
+                for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off);
+                if (lane == 0) a.dsink_partial[((((int64_t)b * n_chunks + chunk) * a.G + g) * a.r + h) * C::NHELP + hh] = v;
+            }
+        }
         return;
     }
 
@@ -341,8 +361,12 @@ __global__ __launch_bounds__(WinCfg::NWAVES * 64, 1) void attn_bwd_window_kernel
     if (n_it > 1) issue(1);
 
     WinPos cur{t0, 0};
-    auto iterate = [&](int it, auto stage_tag) {
-        constexpr int STAGE = decltype(stage_tag)::value;
+    // One copy of the loop body with the LDS stage as a run-time value: a body per stage (stage
+    // offsets as instruction immediates) makes this kernel larger than the instruction cache.
+    int stage = 0;
+    auto iterate = [&](int it) {
+        const int STAGE = stage;
+        stage = stage == NS - 1 ? 0 : stage + 1;
         if (w < 2) { if (it + 1 >= n_it) wait_vmcnt<0>(); else wait_vmcnt<8>(); }
         else if (w == 2 && cur.h == 0) wait_vmcnt<0>();        // the transit copy of the key tile that starts now
         __syncthreads();
@@ -391,11 +415,7 @@ __global__ __launch_bounds__(WinCfg::NWAVES * 64, 1) void attn_bwd_window_kernel
         cur.step(a.r);
     };
 
-    for (int it = 0; it < n_it; it += NS) {
-        iterate(it, std::integral_constant<int, 0>{});
-        if (it + 1 < n_it) iterate(it + 1, std::integral_constant<int, 1>{});
-        if (it + 2 < n_it) iterate(it + 2, std::integral_constant<int, 2>{});
-    }
+    for (int it = 0; it < n_it; ++it) iterate(it);
     __syncthreads();                                           // hands the last dS tile over
     flush();
 }
