@@ -134,6 +134,22 @@ __device__ __forceinline__ void dkdv_tile(uint32_t qsm, uint32_t gsm, uint32_t s
                                           const int (&dbase)[NB], unsigned weff, int row_lim, int krel,
                                           uint32_t ds_lane, const int (&jkey)[NB], uint32_t ds_out = 0) {
     static_assert(!STORE_DS || NB == 1, "the dS store is written for one 32-key block per wavefront");
+    // masked variant, per lane and tile: pair (row r, key) is visible iff 0 <= dbase + r < weff and
+    // r < row_lim.  With r = rc + 4*half (rc a compile-time constant per accumulator register) that is
+    // (unsigned)(dbh + rc) < width with dbh = dbase + 4*half, width = max(0, min(weff, dbh + row_lim - 4*half)):
+    // one add, one compare, one select per element.  Used by the single-pass window kernel, where
+    // two tiles out of three are masked (window layer, S = 16384: -6 %); the dK/dV kernel, whose
+    // masked tiles are the few on the diagonal of a full-causal layer, keeps the plain form (the
+    // folded one costs it 17 registers and 4 % on that layer).
+    int dbh[NB];
+    unsigned width[NB];
+    if (MASKED && STORE_DS) {
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            dbh[nb] = dbase[nb] + 4 * half;
+            width[nb] = (unsigned)max(0, min((int)weff, dbh[nb] + max(row_lim, -8) - 4 * half));
+        }
+    }
     // qsm / gsm: LDS byte addresses of the staged Q and dO tiles; stat_lane: address of this
     // lane's first lse2 value (rows 4*half..), -delta sits kTile floats further on.
     // DOCS (packed rows): ds_lane addresses the staged document starts of the same rows, jkey
@@ -148,15 +164,15 @@ __device__ __forceinline__ void dkdv_tile(uint32_t qsm, uint32_t gsm, uint32_t s
             continue;
         }
         f32x16 s[NB], dp[NB];
-        // the dP accumulators start at -delta of their rows, so the MFMAs deliver dP - delta
+            // the dP accumulators start at -delta of their rows, so the MFMAs deliver dP - delta
 #pragma unroll
-        for (int a4 = 0; a4 < 4; ++a4) {
-            const f32x4 nd = lds_load128f(stat_lane, (kTile + 32 * qb + 8 * a4) * 4);
+            for (int a4 = 0; a4 < 4; ++a4) {
+                const f32x4 nd = lds_load128f(stat_lane, (kTile + 32 * qb + 8 * a4) * 4);
 #pragma unroll
-            for (int nb = 0; nb < NB; ++nb)
+                for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-                for (int e = 0; e < 4; ++e) { s[nb][4 * a4 + e] = 0.0f; dp[nb][4 * a4 + e] = nd[e]; }
-        }
+                    for (int e = 0; e < 4; ++e) { s[nb][4 * a4 + e] = 0.0f; dp[nb][4 * a4 + e] = nd[e]; }
+            }
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
             const bf16x8 aq = ofrag_nat(qsm, lo, qb, ks);
@@ -179,8 +195,13 @@ __device__ __forceinline__ void dkdv_tile(uint32_t qsm, uint32_t gsm, uint32_t s
                     const int i = 4 * a4 + e;
                     float pe = fast_exp2(fmaf(s[nb][i], c, -lv[e]));
                     if (MASKED) {
-                        const int r = 32 * qb + 8 * a4 + 4 * half + e;
-                        bool vis = ((unsigned)(dbase[nb] + r) < weff) & (r < row_lim);
+                        bool vis;
+                        if constexpr (STORE_DS) {
+                            vis = (unsigned)(dbh[nb] + (32 * qb + 8 * a4 + e)) < width[nb];
+                        } else {
+                            const int r = 32 * qb + 8 * a4 + 4 * half + e;
+                            vis = ((unsigned)(dbase[nb] + r) < weff) & (r < row_lim);
+                        }
                         if (DOCS) vis = vis & (jkey[nb] >= (int)dsr[e]);
                         pe = vis ? pe : 0.0f;
                     }
@@ -502,7 +523,7 @@ __device__ __forceinline__ void dq_tile(uint32_t ksm, uint32_t vsm, const TileLa
             }
         }
 #pragma unroll
-        for (int qb = 0; qb < NQB; ++qb)
+        for (int qb = 0; qb < NQB; ++qb) {
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 float pe = fast_exp2(fmaf(s[qb][i], c, -lse2[qb]));
@@ -513,6 +534,7 @@ __device__ __forceinline__ void dq_tile(uint32_t ksm, uint32_t vsm, const TileLa
                 }
                 dp[qb][i] = qb == 0 ? pe * dp[qb][i] : pe * (dp[qb][i] + dlt[qb]);        // dlt holds -delta
             }
+        }
 #pragma unroll
         for (int u = 0; u < 2; ++u) {
             bf16x8 akt[2];

@@ -92,6 +92,24 @@ __device__ __forceinline__ float xhalf_sum(float x) {
 }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
+// Visibility test of the kernels whose lanes are query rows and whose accumulator registers are
+// keys (forward, dQ).  Key r of the tile is visible to the lane iff 0 <= dbase - r < wl and
+// r < key_lim, where dbase = (lane's query position) - (first key of the tile), hugely negative
+// for a dead row.  Register i of a 32-key block holds key r = rc + 4*half with rc a compile-time
+// constant, so with everything lane-dependent folded into two values per tile the test is
+// (unsigned)(base - rc) < width: one subtract, one compare, one select per element.
+struct KeyMask { int base; unsigned width; };
+__device__ __forceinline__ KeyMask make_key_mask(int dbase, unsigned wl, int key_lim, int half) {
+    const int dbh = dbase - 4 * half;
+    const int kl = min(max(key_lim, -8), 72) - 4 * half;     // only its relation to 0..63 matters
+    const int lo = max(0, dbh - kl + 1);                       // dbase - r >= lo  <=>  r < key_lim (and r <= dbase)
+    KeyMask m;
+    m.base = dbh - lo;
+    m.width = (unsigned)max(0, (int)wl - lo);
+    return m;
+}
+__device__ __forceinline__ bool key_visible(const KeyMask &m, int rc) { return (unsigned)(m.base - rc) < m.width; }
+
 // B fragment from C registers 8*u .. 8*u+7: converted to bf16 they hold, in k-slot order, exactly
 // the rows that a transposed A fragment (ofrag_tr) of the same 16-row step holds.
 __device__ __forceinline__ bf16x8 cfrag(const f32x16 &c, int u) {

@@ -59,15 +59,13 @@ __device__ __forceinline__ void fwd_tile(uint32_t ksm, uint32_t vsm, const TileL
 #pragma unroll
     for (int qb = 0; qb < NQB; ++qb) {
         if (MASKED) {
+            const KeyMask km = make_key_mask(dbase[qb], wl[qb], key_lim, half);
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
                 if (!dead[kb]) {
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        const int r = 32 * kb + crow(i, half);
-                        const bool vis = ((unsigned)(dbase[qb] - r) < wl[qb]) & (r < key_lim);
-                        s[kb][qb][i] = vis ? s[kb][qb][i] : -INFINITY;
-                    }
+                    for (int i = 0; i < 16; ++i)
+                        s[kb][qb][i] = key_visible(km, 32 * kb + 8 * (i >> 2) + (i & 3)) ? s[kb][qb][i] : -INFINITY;
                 }
         }
         // two independent reduction chains keep the VALU pipelined
