@@ -5,18 +5,28 @@ A "step" is one forward + backward of a single GPT-OSS-20B attention layer
 (64 query heads over 8 KV heads, head_dim 64, bf16, B=1) on synthetic N(0,1)
 inputs already resident in HBM.  The headline workload is the full-causal layer
 at S=16384; the same shape with sliding window 128 is timed next to it to report
-the tile-skipping speedup.
+the tile-skipping speedup, and configs 2 (S=4096) and 4 (padded batch of 4) are
+timed as extra keys.
 
 Prints ONE JSON line.  `value` is algorithmic TFLOP/s of fwd+bwd
 (FLOPs = 14 * D * pairs * B * H, pairs = S(S+1)/2), `roofline` describes the
 dominant kernel, `cpu_baseline` is the eager fp32 restatement timed on the host
 cores on a bounded sample of the same workload.
+
+Two more modes serve the committed profiles:
+  --layers full|window   run one layer type only (what rocprofv3 is pointed at)
+  --summarize ...        turn rocprofv3's result databases into profiles/*.md and
+                         the HBM-traffic record the `roofline.traffic` field is read from
 """
 from __future__ import annotations
 
 import argparse
+import collections
+import ctypes
+import hashlib
 import json
 import os
+import platform
 import statistics
 import sys
 import time
@@ -26,11 +36,34 @@ sys.path.insert(0, ROOT)
 
 PEAK_BF16_TFLOPS = 2516.6   # MI355X dense bf16 MFMA peak
 PEAK_HBM_GBS = 8000.0
-DKDV_HBM_BYTES_S16K = int((702233.8 * 2.0 + 32768.0) * 1024)   # measured, see profiles/
+TRAFFIC_JSON = os.path.join(ROOT, "profiles", "hbm_traffic_S16384.json")
+CSRC = os.path.join(ROOT, "oregon_gpt_oss_patching_amd", "csrc")
 
 
 def pairs(s, w):
     return s * (s + 1) // 2 if not w or w >= s else w * s - w * (w - 1) // 2
+
+
+def source_hash():
+    """Identifies the kernel sources a profile was taken with."""
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(CSRC)):
+        if name.endswith((".h", ".hip")):
+            h.update(name.encode())
+            h.update(open(os.path.join(CSRC, name), "rb").read())
+    return h.hexdigest()[:16]
+
+
+def recorded_traffic(kernel, layer):
+    """HBM bytes per launch of `kernel` from the committed counter record, or None when the
+    record was taken with other kernel sources (or does not exist)."""
+    try:
+        rec = json.load(open(TRAFFIC_JSON))
+    except (OSError, ValueError):
+        return None
+    if rec.get("source_hash") != source_hash():
+        return None
+    return rec.get("layers", {}).get(layer, {}).get(kernel, {}).get("hbm_bytes")
 
 
 def device_info():
@@ -45,6 +78,54 @@ def device_info():
     return info
 
 
+def make_inputs(seed, b, h, g, s, d, dtype):
+    """Seeded N(0,1) tensors drawn on the CPU in the order Q, K, V, sinks, dO (the order the
+    parity tests use), rounded to `dtype`."""
+    import torch
+    gen = torch.Generator(device="cpu").manual_seed(seed)
+    q = torch.randn(b, h, s, d, generator=gen).to(dtype)
+    k = torch.randn(b, g, s, d, generator=gen).to(dtype)
+    v = torch.randn(b, g, s, d, generator=gen).to(dtype)
+    sinks = torch.randn(h, generator=gen).to(dtype)
+    d_out = torch.randn(b, s, h, d, generator=gen).to(dtype)
+    return q, k, v, sinks, d_out
+
+
+class Problem:
+    """Inputs, outputs and the pre-built parameter block of one layer call, so that a timed
+    region is only the library launches."""
+
+    def __init__(self, seed, b, s, window, seqlens=None, h=64, g=8, d=64, scale=0.125):
+        import torch
+        from oregon_gpt_oss_patching_amd import _lib
+        from oregon_gpt_oss_patching_amd import attention_kernel as ak
+        dev = torch.device("cuda:0")
+        self.b, self.s, self.h, self.g, self.d, self.window = b, s, h, g, d, window
+        q, k, v, sinks, d_out = (t.to(dev) for t in make_inputs(seed, b, h, g, s, d, torch.bfloat16))
+        # V as the model delivers it: a transposed view of the (B, S, G, D) projection output
+        v = v.transpose(1, 2).contiguous().transpose(1, 2)
+        o = torch.empty((b, s, h, d), dtype=q.dtype, device=dev)
+        lse = torch.empty((b, h, s), dtype=torch.float32, device=dev)
+        dq, dk, dv = torch.empty_like(q), torch.empty(k.shape, dtype=k.dtype, device=dev), torch.empty(k.shape, dtype=k.dtype, device=dev)
+        dsinks = torch.empty((h,), dtype=torch.float32, device=dev)
+        s32 = sinks.float().contiguous()
+        sl = None if seqlens is None else torch.tensor(seqlens, dtype=torch.int32, device=dev)
+        p = ak._base_params(q, k, v, s32, sl, scale, window, 0)
+        # backward scratch, sized by the library
+        delta = torch.empty((_lib.load().gptoss_attn_workspace_bytes(ctypes.byref(p)) // 4,), dtype=torch.float32, device=dev)
+        p.o, p.lse = o.data_ptr(), lse.data_ptr()
+        ak._set(p.o_stride, ak._strides_bhs(o, "bshd"))
+        p.d_o = d_out.data_ptr()
+        ak._set(p.do_stride, ak._strides_bhs(d_out, "bshd"))
+        p.dq, p.dk, p.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
+        ak._set(p.dq_stride, ak._strides_bhs(dq, "bhsd"))
+        ak._set(p.dk_stride, ak._strides_bhs(dk, "bhsd"))
+        ak._set(p.dv_stride, ak._strides_bhs(dv, "bhsd"))
+        p.delta, p.dsinks = delta.data_ptr(), dsinks.data_ptr()
+        self.params = p
+        self.keep = (q, k, v, d_out, o, lse, dq, dk, dv, delta, dsinks, s32, sl)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -57,7 +138,14 @@ def main():
                     help="which layer types to run (profiling runs use one, so per-kernel averages are unmixed)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run a plain 1 GiB device copy, the known-size kernel that HBM byte counters are scaled by")
+    ap.add_argument("--summarize", nargs="+", metavar="DIR",
+                    help="rocprofv3 output directories (each holding one *_results.db) of runs made with --layers L "
+                         "--copy-calibration; writes the summary given by --out-md and updates the traffic record")
+    ap.add_argument("--summary-layer", choices=("full", "window"))
+    ap.add_argument("--out-md")
     args = ap.parse_args()
+    if args.summarize:
+        return summarize(args.summarize, args.summary_layer, args.out_md)
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the attention op has no cross-GPU "
               "exchange; every box here has one GPU). Run with --gpus 1.", file=sys.stderr)
@@ -65,40 +153,11 @@ def main():
 
     import torch
     from oregon_gpt_oss_patching_amd import _lib
-    from oregon_gpt_oss_patching_amd import attention_kernel as ak
-    from oracle import eager_ref as E
 
     assert torch.cuda.is_available(), "bench.py needs the GPU"
     _lib.load()
     dev = torch.device("cuda:0")
     B, H, G, D, S = 1, 64, 8, 64, args.seq
-    scale = 0.125
-    q, k, v, sinks, d_out = (t.to(dev) for t in E.make_inputs(3, B, H, G, S, D, torch.bfloat16))
-    # V as the model delivers it: a transposed view of the (B, S, G, D) projection output
-    v = v.transpose(1, 2).contiguous().transpose(1, 2)
-
-    def make_params(window):
-        """Pre-built parameter block + output buffers, so the timed region is only the launches."""
-        o = torch.empty((B, S, H, D), dtype=q.dtype, device=dev)
-        lse = torch.empty((B, H, S), dtype=torch.float32, device=dev)
-        dq, dk, dv = torch.empty_like(q), torch.empty(k.shape, dtype=k.dtype, device=dev), torch.empty(k.shape, dtype=k.dtype, device=dev)
-        dsinks = torch.empty((H,), dtype=torch.float32, device=dev)
-        s32 = sinks.float().contiguous()
-        p = ak._base_params(q, k, v, s32, None, scale, window, 0)
-        # backward scratch ([-delta; lse*log2e], plus dK/dV partials when S is short), sized by the library
-        delta = torch.empty((_lib.load().gptoss_attn_workspace_bytes(p) // 4,), dtype=torch.float32, device=dev)
-        p.o, p.lse = o.data_ptr(), lse.data_ptr()
-        ak._set(p.o_stride, ak._strides_bhs(o, "bshd"))
-        p.d_o = d_out.data_ptr()
-        ak._set(p.do_stride, ak._strides_bhs(d_out, "bshd"))
-        p.dq, p.dk, p.dv = dq.data_ptr(), dk.data_ptr(), dv.data_ptr()
-        ak._set(p.dq_stride, ak._strides_bhs(dq, "bhsd"))
-        ak._set(p.dk_stride, ak._strides_bhs(dk, "bhsd"))
-        ak._set(p.dv_stride, ak._strides_bhs(dv, "bhsd"))
-        p.delta, p.dsinks = delta.data_ptr(), dsinks.data_ptr()
-        keep = (o, lse, dq, dk, dv, delta, dsinks, s32)
-        return p, keep
-
     stream = torch.cuda.current_stream(dev)
     sptr = stream.cuda_stream
 
@@ -129,8 +188,9 @@ def main():
         ts = [a.elapsed_time(b) for a, b in evs]
         return statistics.mean(ts)
 
-    p_full, keep_full = make_params(0)
-    p_win, keep_win = make_params(128)
+    full = Problem(3, B, S, 0)
+    win = Problem(3, B, S, 128)
+    p_full, p_win = full.params, win.params
 
     # A fresh process starts with the GPU at idle clocks and cold instruction caches; a fixed
     # number of untimed steps before the W warm-up steps keeps short runs (small W) from timing
@@ -159,8 +219,9 @@ def main():
 
     kern = {}
     for tag, p in (("full", p_full), ("win128", p_win)):
-        # the separate backward entry points, then the combined one (gptoss_attn_bwd), whose dQ kernel
-        # computes the row statistics itself and which therefore runs no preprocess kernel
+        # the separate backward entry points, then the combined one (gptoss_attn_bwd): for the full-causal layer
+        # its dQ kernel computes the row statistics itself (no preprocess kernel), for the sliding-window layer it
+        # is the single-pass kernel
         for name in ("gptoss_attn_fwd", "gptoss_attn_bwd_preprocess", "gptoss_attn_bwd_dkdv", "gptoss_attn_bwd_dq",
                      "gptoss_attn_bwd"):
             kern[f"{tag}.{name[12:]}"] = round(time_kernel(name, p), 4)
@@ -169,11 +230,28 @@ def main():
     fl_total = 7 * unit
     tflops = fl_total / (ms_full * 1e-3) / 1e12
     unit_w = 2 * D * pairs(S, 128) * B * H
-    bytes_total = 2 * B * S * D * (2 * H + 2 * G) + 4 * B * H * S + 2 * B * S * D * (4 * H + 4 * G) + 12 * B * H * S
+    bytes_fwd = 2 * B * S * D * (2 * H + 2 * G) + 4 * B * H * S
+    bytes_bwd = 2 * B * S * D * (4 * H + 4 * G) + 12 * B * H * S
+    bytes_total = bytes_fwd + bytes_bwd
 
     # dominant kernel: dkdv computes S, dP, dV, dK = 4 of the 7 algorithmic GEMMs
     dkdv_ms = kern["full.bwd_dkdv"]
     dkdv_tflops = 4 * unit / (dkdv_ms * 1e-3) / 1e12
+    win_bwd_ms = kern["win128.bwd"]
+
+    # configs 2 and 4 of the reference's benchmark list, fwd + bwd through the same entry points
+    other = {}
+    gen = torch.Generator(device="cpu").manual_seed(4)
+    lens4 = torch.randint(1024, 4097, (4,), generator=gen).tolist()
+    for tag, prob, valid_pairs in (
+            ("config2.full", Problem(2, 1, 4096, 0), pairs(4096, 0)),
+            ("config2.win128", Problem(2, 1, 4096, 128), pairs(4096, 128)),
+            ("config4.full", Problem(4, 4, 4096, 0, lens4), sum(pairs(n, 0) for n in lens4)),
+            ("config4.win128", Problem(4, 4, 4096, 128, lens4), sum(pairs(n, 128) for n in lens4))):
+        ms = time_steps(prob.params, 20, 5)
+        other[tag] = {"ms_per_step": round(ms, 4), "tflops": round(14 * D * valid_pairs * H / (ms * 1e-3) / 1e12, 1)}
+        del prob
+    other["config4.lengths"] = lens4
 
     out = {
         "metric": "attn fwd+bwd TFLOP/s & % bf16 MFMA peak, GPT-OSS-20B shape, S=16K, 1 GPU",
@@ -196,37 +274,184 @@ def main():
                       "algorithmic_GBs": round(bytes_total / (ms_win * 1e-3) / 1e9, 1),
                       "frac_hbm_peak": round(bytes_total / (ms_win * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
                       "speedup_vs_full": round(ms_full / ms_win, 2),
-                      "speedup_target": S / 256 * 0.5},
+                      "speedup_target": S / 256 * 0.5,
+                      # the single-pass backward kernel against the HBM roofline: algorithmic backward bytes
+                      # (read Q, O, dO, K, V, lse; write dQ, dK, dV) over its launch time
+                      "bwd_kernel": {"bound": "hbm", "kernel": "attn_bwd_window_kernel",
+                                     "achieved": round(bytes_bwd / (win_bwd_ms * 1e-3) / 1e9, 1), "peak": PEAK_HBM_GBS,
+                                     "unit": "GB/s", "frac": round(bytes_bwd / (win_bwd_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+                                     "traffic": recorded_traffic("attn_bwd_window_kernel", "window") if S == 16384 else None}},
         "kernel_ms": kern,
+        "other_configs": other,
         "device": device_info(),
         "roofline": {"bound": "mfma", "kernel": "attn_bwd_dkdv_kernel (full causal)",
                      "achieved": round(dkdv_tflops, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(dkdv_tflops / PEAK_BF16_TFLOPS, 4),
-                     # HBM bytes per launch of this kernel at S=16384 from rocprofv3 --pmc FETCH_SIZE (x2.0) and
-                     # WRITE_SIZE (x1.0), factors from a plain 1 GiB copy kernel; only valid for the default shape
-                     "traffic": DKDV_HBM_BYTES_S16K if S == 16384 else None},
+                     # HBM bytes per launch of this kernel at S=16384 from the committed rocprofv3 counter record
+                     # (FETCH_SIZE and WRITE_SIZE scaled by a plain 1 GiB copy); null when that record was taken
+                     # with other kernel sources
+                     "traffic": recorded_traffic("attn_bwd_dkdv_kernel", "full") if S == 16384 else None},
     }
 
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(E, args.cpu_seq, D, scale)
+        out["cpu_baseline"] = cpu_baseline(args.cpu_seq, D, 0.125)
     print(json.dumps(out))
 
 
-def cpu_baseline(E, s, d, scale):
-    """Eager fp32 restatement (forward + autograd backward) on the host cores, on a
-    bounded sample: two query heads sharing one KV head of the full-causal layer."""
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return platform.processor() or "unknown"
+
+
+def cpu_baseline(s, d, scale):
+    """Eager fp32 restatement (forward + autograd backward) on the host cores, on a bounded
+    sample: two query heads sharing one KV head of the full-causal layer.  Threads: what torch
+    was given (OMP_NUM_THREADS / the CPU share of the box), never more than the host reports."""
     import torch
-    cores = min(os.cpu_count() or 1, 16)
+    from oracle import eager_ref as E
+    host = os.cpu_count() or 1
+    cores = max(1, min(torch.get_num_threads(), host))
     torch.set_num_threads(cores)
-    heads = 2
-    q, k, v, sinks, d_out = E.make_inputs(3, 1, heads, 1, s, d, torch.float32)
-    t0 = time.perf_counter()
-    E.eager_attention_grads(q, k, v, sinks, d_out, scale, None)
-    dt = time.perf_counter() - t0
-    fl = 14 * d * pairs(s, 0) * heads
-    return {"value": round(fl / dt / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "kind": "port",
-            "sample": f"{heads} of 64 query heads (one KV head) of the S={s} full-causal layer, eager fp32 fwd + autograd bwd, "
-                      f"{dt:.1f} s wall; algorithmic FLOPs counted as for the GPU"}
+    heads, calls = 4, 2
+    warm = E.make_inputs(1, 1, heads, 1, 1024, d, torch.float32)
+    E.eager_attention_grads(*warm, scale, None)                      # warm-up: thread pool, allocator
+    dt = 0.0
+    for i in range(calls):
+        q, k, v, sinks, d_out = E.make_inputs(3 + i, 1, heads, 1, s, d, torch.float32)
+        t0 = time.perf_counter()
+        E.eager_attention_grads(q, k, v, sinks, d_out, scale, None)
+        dt += time.perf_counter() - t0
+        del q, k, v, sinks, d_out
+    fl = 14 * d * pairs(s, 0) * heads * calls
+    return {"value": round(fl / dt / 1e12, 4), "unit": "TFLOP/s", "cores": cores, "host_cpu_count": host,
+            "cpu_model": cpu_model(), "kind": "port",
+            "sample": f"{heads * calls} of 64 query heads ({calls} calls of {heads} heads on one KV head) of the S={s} full-causal "
+                      f"layer, eager fp32 fwd + autograd bwd, {dt:.1f} s wall after one small warm-up call; algorithmic FLOPs "
+                      f"counted as for the GPU"}
+
+
+# ---- rocprofv3 summaries -----------------------------------------------------------------------
+
+def _read_rocpd(path):
+    """Per-kernel call count, average duration and summed counters of one rocprofv3 result database."""
+    import sqlite3
+    db = sqlite3.connect(path)
+    cur = db.cursor()
+    tables = [r[0] for r in cur.execute("select name from sqlite_master where type='table'")]
+
+    def table(prefix):
+        return next(t for t in tables if t.startswith(prefix))
+    names = {r[0]: r[1] for r in cur.execute(f"select id, kernel_name from {table('rocpd_info_kernel_symbol')}")}
+    rows = list(cur.execute(f"select kernel_id, start, end, event_id from {table('rocpd_kernel_dispatch')} order by start"))
+    pmc = {}
+    try:
+        pn = {r[0]: r[1] for r in cur.execute(f"select id, name from {table('rocpd_info_pmc')}")}
+        for ev, pid, val in cur.execute(f"select event_id, pmc_id, value from {table('rocpd_pmc_event')}"):
+            pmc.setdefault(ev, collections.Counter())[pn.get(pid, str(pid))] += val
+    except (StopIteration, sqlite3.Error):
+        pass
+    agg = collections.OrderedDict()
+    for kid, st, en, ev in rows:
+        n = _short_name(names.get(kid, str(kid)))
+        a = agg.setdefault(n, {"calls": 0, "ns": 0, "min_ns": 1 << 62, "pmc": collections.Counter(), "per_call": []})
+        a["calls"] += 1
+        a["ns"] += en - st
+        a["min_ns"] = min(a["min_ns"], en - st)
+        a["pmc"].update(pmc.get(ev, {}))
+        a["per_call"].append(dict(pmc.get(ev, {})))
+    return agg
+
+
+_DEMANGLED = {}
+
+
+def _short_name(mangled):
+    """Kernel name without namespace, template arguments, parameter list and the .kd suffix."""
+    import shutil
+    import subprocess
+    if mangled not in _DEMANGLED:
+        name = mangled[:-3] if mangled.endswith(".kd") else mangled
+        tool = shutil.which("c++filt") or shutil.which("llvm-cxxfilt")
+        if tool and name.startswith("_Z"):
+            try:
+                name = subprocess.run([tool, name], capture_output=True, text=True, timeout=10).stdout.strip() or name
+            except (OSError, subprocess.SubprocessError):
+                pass
+        name = name.replace("void ", "").split("(")[0].split("<")[0]
+        _DEMANGLED[mangled] = name.split("::")[-1]
+    return _DEMANGLED[mangled]
+
+
+def summarize(dirs, layer, out_md):
+    """Reads the *_results.db of each directory, prints / writes a text summary and records the
+    HBM bytes per launch (FETCH_SIZE, WRITE_SIZE scaled by what the 1 GiB calibration copy shows)."""
+    assert layer and out_md, "--summarize needs --summary-layer and --out-md"
+    sections, fetch, write, dur = [], {}, {}, {}
+    for d in dirs:
+        dbs = [os.path.join(r, f) for r, _, fs in os.walk(d) for f in fs if f.endswith("_results.db")]
+        assert dbs, f"no *_results.db under {d}"
+        agg = _read_rocpd(dbs[0])
+        total = sum(a["ns"] for a in agg.values()) or 1
+        lines = []
+        for n, a in sorted(agg.items(), key=lambda kv: -kv[1]["ns"]):
+            extra = " ".join(f"{k}/call={v / a['calls']:.1f}" for k, v in sorted(a["pmc"].items()))
+            lines.append(f"{n:40s} calls {a['calls']:3d} avg {a['ns'] / a['calls'] / 1e3:9.1f} us  min {a['min_ns'] / 1e3:9.1f}  "
+                         f"{100 * a['ns'] / total:5.1f}%  {extra}".rstrip())
+            if "FETCH_SIZE" in a["pmc"]:
+                fetch[n] = a["pmc"]["FETCH_SIZE"] / a["calls"]
+            if "WRITE_SIZE" in a["pmc"]:
+                write[n] = a["pmc"]["WRITE_SIZE"] / a["calls"]
+            if not a["pmc"]:
+                dur[n] = a["ns"] / a["calls"] / 1e3
+        sections.append((os.path.basename(os.path.normpath(d)), lines))
+    # calibration: each large call of the copy kernel reads 1 GiB and writes 1 GiB (small calls of the same
+    # kernel, e.g. torch's own housekeeping copies, are left out: they move a few KiB)
+    f_fac = w_fac = None
+    for d in dirs:
+        dbs = [os.path.join(r, f) for r, _, fs in os.walk(d) for f in fs if f.endswith("_results.db")]
+        for n, a in _read_rocpd(dbs[0]).items():
+            if "copyBuffer" not in n:
+                continue
+            for key in ("FETCH_SIZE", "WRITE_SIZE"):
+                big = [c[key] for c in a["per_call"] if c.get(key, 0) > (1 << 18)]
+                if big:
+                    fac = (1 << 20) / statistics.median(big)
+                    if key == "FETCH_SIZE":
+                        f_fac = round(fac, 3)
+                    else:
+                        w_fac = round(fac, 3)
+    kernels = {}
+    for n in fetch:
+        if n in write and f_fac and w_fac and n.startswith("attn_"):
+            kernels[n] = {"avg_us": round(dur.get(n, 0.0), 1), "fetch_kib": round(fetch[n], 1), "write_kib": round(write[n], 1),
+                          "hbm_bytes": int((fetch[n] * f_fac + write[n] * w_fac) * 1024)}
+    text = [f"Source hash {source_hash()}; calibration factors from the 1 GiB copy: FETCH_SIZE x {f_fac}, WRITE_SIZE x {w_fac}.", ""]
+    for name, lines in sections:
+        text += [f"## {name}", "", "```"] + lines + ["```", ""]
+    text += ["## HBM bytes per launch (FETCH_SIZE x factor + WRITE_SIZE x factor)", "", "```"]
+    text += [f"{n:40s} {k['hbm_bytes'] / 1e6:10.1f} MB" for n, k in kernels.items()] + ["```", ""]
+    body = "\n".join(text)
+    if os.path.exists(out_md) and "<!-- generated below -->" in open(out_md).read():
+        head = open(out_md).read().split("<!-- generated below -->")[0]
+        body = head + "<!-- generated below -->\n\n" + body
+    open(out_md, "w").write(body)
+    rec = {}
+    if os.path.exists(TRAFFIC_JSON):
+        try:
+            rec = json.load(open(TRAFFIC_JSON))
+        except ValueError:
+            rec = {}
+    if rec.get("source_hash") != source_hash():
+        rec = {"source_hash": source_hash(), "workload": "B=1 S=16384 H=64 G=8 D=64 bf16", "layers": {}}
+    rec["calibration"] = {"fetch_factor": f_fac, "write_factor": w_fac}
+    rec["layers"][layer] = kernels
+    json.dump(rec, open(TRAFFIC_JSON, "w"), indent=1, sort_keys=True)
+    print(body)
 
 
 if __name__ == "__main__":

@@ -113,6 +113,73 @@ __device__ __forceinline__ void fwd_tile(uint32_t ksm, uint32_t vsm, const TileL
     }
 }
 
+// The same tile with the softmax reference FROZEN: p = exp2(s*c + nm) with nm = -m, the lane's
+// reference as the first tile of the row left it (the row maximum over that tile, or the sink
+// logit if that is larger).  This is the reference's online softmax (attention_kernel.py:79-96)
+// with the running maximum no longer updated: O = sum(p v) / (sum p + exp(sink - m)) is the same
+// quotient for any m as long as nothing overflows, so after the first tile the key loop needs no
+// row maximum, no comparison and no rescaling of O (in a sliding-window layer nearly every one
+// of a row's three tiles moves the maximum and pays for that rescaling).  A row whose later
+// logits climb more than about 95 (natural units) above its reference would overflow; the
+// kernel detects that after the loop and repeats the workgroup with the exact step (fwd_tile)
+// on every tile.  Logits far below the reference underflow to p = 0, which is what they
+// contribute.  The row sum stays an fp32 sum of the unrounded probabilities, so lse is as
+// exact as in fwd_tile.
+template <bool MASKED, int NQB>
+__device__ __forceinline__ void fwd_tile_lean(uint32_t ksm, uint32_t vsm, const TileLaneOffsets &lo, const bf16x8 (&qf)[NQB][4],
+                                              f32x16 (&o)[NQB][2], const float (&nm)[NQB], float (&l)[NQB], float c, int lane,
+                                              const int (&dbase)[NQB], const unsigned (&wl)[NQB], unsigned weff, int key_lim,
+                                              int wrel) {
+    const int half = lane >> 5;
+#pragma unroll
+    for (int kb = 0; kb < 2; ++kb) {
+        if (MASKED && ((32 * kb > wrel + 32 * NQB - 1) || (32 * kb + 31 < wrel - (int)weff + 1) || (32 * kb >= key_lim))) continue;
+        f32x16 s[NQB];
+#pragma unroll
+        for (int qb = 0; qb < NQB; ++qb)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) s[qb][i] = 0.0f;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            const bf16x8 ak = ofrag_nat(ksm, lo, kb, ks);
+#pragma unroll
+            for (int qb = 0; qb < NQB; ++qb) s[qb] = mfma_bf16(ak, qf[qb][ks], s[qb]);
+        }
+#pragma unroll
+        for (int qb = 0; qb < NQB; ++qb) {
+            KeyMask km{0, 0u};
+            if (MASKED) km = make_key_mask(dbase[qb], wl[qb], key_lim, half);
+            float rs0 = 0.0f, rs1 = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 16; i += 2) {
+                float t0 = fmaf(s[qb][i], c, nm[qb]), t1 = fmaf(s[qb][i + 1], c, nm[qb]);
+                if (MASKED) {
+                    t0 = key_visible(km, 32 * kb + 8 * (i >> 2) + (i & 3)) ? t0 : -INFINITY;
+                    t1 = key_visible(km, 32 * kb + 8 * (i >> 2) + (i & 3) + 1) ? t1 : -INFINITY;
+                }
+                const float e0 = fast_exp2(t0), e1 = fast_exp2(t1);
+                s[qb][i] = e0;
+                s[qb][i + 1] = e1;
+                rs0 += e0;
+                rs1 += e1;
+            }
+            l[qb] += rs0 + rs1;
+        }
+#pragma unroll
+        for (int u = 0; u < 2; ++u) {
+            bf16x8 av[2];
+#pragma unroll
+            for (int dblk = 0; dblk < 2; ++dblk) av[dblk] = ofrag_tr(vsm, lo, kb, u, dblk);
+#pragma unroll
+            for (int qb = 0; qb < NQB; ++qb) {
+                const bf16x8 pf = cfrag(s[qb], u);
+#pragma unroll
+                for (int dblk = 0; dblk < 2; ++dblk) o[qb][dblk] = mfma_bf16(av[dblk], pf, o[qb][dblk]);
+            }
+        }
+    }
+}
+
 template <int HPB, int NQB>
 __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_fwd_kernel(const KArgs a) {
     constexpr int QSUB = 4 / HPB;      // row slabs per workgroup
@@ -188,16 +255,9 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_fwd_kernel(const
 
     const float c = a.scale_log2;
     const float sink2 = (a.sinks ? a.sinks[head] : 0.0f) * kLog2e;
-    float m[NQB], l[NQB];  // running max (log2 domain, starts at the sink logit, ref :53) and
+    float m[NQB], l[NQB];  // softmax reference (log2 domain, starts at the sink logit, ref :53) and
                            // this lane's share of the running sum (own keys only)
     f32x16 o[NQB][2];
-#pragma unroll
-    for (int qb = 0; qb < NQB; ++qb) {
-        m[qb] = sink2;
-        l[qb] = 0.0f;
-#pragma unroll
-        for (int i = 0; i < 16; ++i) { o[qb][0][i] = 0.0f; o[qb][1][i] = 0.0f; }
-    }
 
     const TileLaneOffsets lo = make_tile_offsets(lane);
     const uint32_t smem_base = lds_addr(&smem[0][0][0]);
@@ -205,9 +265,9 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_fwd_kernel(const
     // K / V tiles are requested in order; the pointers to the next tile's first row advance by
     // one tile per request.  Only a tile that sticks out of the tensor takes the clamping copy.
     const AsyncLaneOffsets klane = make_async_offsets(a.ks.s, lane, w), vlane = make_async_offsets(a.vs.s, lane, w);
-    const bf16 *ktile = kbase + (int64_t)t_lo * kTile * a.ks.s, *vtile = vbase + (int64_t)t_lo * kTile * a.vs.s;
-    int next_row0 = t_lo * kTile;
-    auto issue = [&](int it) {
+    const bf16 *ktile = kbase, *vtile = vbase;
+    int next_row0 = 0;
+    auto issue = [&](int it) __attribute__((always_inline)) {
         const int stage = it % NS;
         if (next_row0 + kTile <= a.Skv) {
             tile_async_inner(smem[stage][0], ktile, klane, w);
@@ -222,12 +282,33 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_fwd_kernel(const
     };
     constexpr int kLoadsPerIt = 4;     // vector-memory instructions one wavefront issues per iteration
 
-    auto iterate = [&](int it, auto stage_tag) {
-        constexpr int STAGE = decltype(stage_tag)::value;
+    // (re)starts the walk over the workgroup's key tiles
+    auto reset = [&]() __attribute__((always_inline)) {
+        ktile = kbase + (int64_t)t_lo * kTile * a.ks.s;
+        vtile = vbase + (int64_t)t_lo * kTile * a.vs.s;
+        next_row0 = t_lo * kTile;
+#pragma unroll
+        for (int qb = 0; qb < NQB; ++qb) {
+            m[qb] = sink2;
+            l[qb] = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) { o[qb][0][i] = 0.0f; o[qb][1][i] = 0.0f; }
+        }
+        if (n_it > 0) issue(0);
+        if (n_it > 1) issue(1);
+    };
+    // the synchronisation every iteration starts with: this tile's copies have landed in every
+    // wavefront, the stage two tiles ahead is free
+    auto arrive = [&](int it) __attribute__((always_inline)) {
         if (it + 1 < n_it) wait_vmcnt<kLoadsPerIt>(); else wait_vmcnt<0>();
         __syncthreads();
         if (it + 2 < n_it) issue(it + 2);
-        const uint32_t ksm = smem_base + STAGE * (2 * kStageTileBytes), vsm = ksm + kStageTileBytes;
+    };
+    // One key tile from the LDS stage at ksm.  EXACT: the online-softmax step that moves the
+    // reference m (fwd_tile); otherwise m stays where it is (fwd_tile_lean).
+    auto tile_step = [&](int it, uint32_t ksm, auto exact_tag) __attribute__((always_inline)) {
+        constexpr bool EXACT = decltype(exact_tag)::value;
+        const uint32_t vsm = ksm + kStageTileBytes;
         const int n0 = (t_lo + it) * kTile;
         // tile classification for this wavefront: skip / interior / needs mask
         const bool skip = !active || n0 > wpos1 || (n0 + kTile - 1) < (wpos0 - weff + 1) || wpos1 < wpos0 ||
@@ -235,22 +316,67 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_fwd_kernel(const
         if (skip) return;
         const bool interior = (n0 + kTile - 1 <= wpos0) && (n0 > wpos1 - weff) && (n0 + kTile <= kv_len) &&
                               (a.q_offset + qw0 + WM - 1 <= wpos1) && (n0 >= ds_w1);
-        if (interior) {
-            fwd_tile<false, NQB>(ksm, vsm, lo, qf, o, m, l, c, lane, pq, wl, 0u, 0, 0);
-        } else {
-            int dbase[NQB];
+        int dbase[NQB];
 #pragma unroll
-            for (int qb = 0; qb < NQB; ++qb) dbase[qb] = pq[qb] - n0;   // stays hugely negative for dead rows
-            fwd_tile<true, NQB>(ksm, vsm, lo, qf, o, m, l, c, lane, dbase, wl, (unsigned)weff, kv_len - n0, wpos0 - n0);
+        for (int qb = 0; qb < NQB; ++qb) dbase[qb] = pq[qb] - n0;   // stays hugely negative for dead rows
+        if constexpr (EXACT) {
+            if (interior) fwd_tile<false, NQB>(ksm, vsm, lo, qf, o, m, l, c, lane, pq, wl, 0u, 0, 0);
+            else fwd_tile<true, NQB>(ksm, vsm, lo, qf, o, m, l, c, lane, dbase, wl, (unsigned)weff, kv_len - n0, wpos0 - n0);
+        } else {
+            float nm[NQB];
+#pragma unroll
+            for (int qb = 0; qb < NQB; ++qb) nm[qb] = -m[qb];
+            if (interior) fwd_tile_lean<false, NQB>(ksm, vsm, lo, qf, o, nm, l, c, lane, pq, wl, 0u, 0, 0);
+            else fwd_tile_lean<true, NQB>(ksm, vsm, lo, qf, o, nm, l, c, lane, dbase, wl, (unsigned)weff, kv_len - n0, wpos0 - n0);
         }
     };
+    // Long full-causal rows (64-row wavefronts) freeze the reference after their first tile.  The
+    // 32-row wavefronts of sliding-window layers keep the exact step on all of their three tiles:
+    // measured, the frozen form does not pay there (0.099 -> 0.103 ms at S = 16384), and with so
+    // few keys per row a dominant key met after the first tile (weights above 1 in the numerator,
+    // bf16-rounded there but not in the denominator) shows in dQ of sharply peaked rows.
+    constexpr bool kFreeze = NQB == 2;
+    auto lean_step = [&](int it, auto stage_tag) __attribute__((always_inline)) {
+        constexpr int STAGE = decltype(stage_tag)::value;
+        arrive(it);
+        tile_step(it, smem_base + STAGE * (2 * kStageTileBytes), std::integral_constant<bool, !kFreeze>{});
+    };
 
-    if (n_it > 0) issue(0);
-    if (n_it > 1) issue(1);
-    for (int it = 0; it < n_it; it += NS) {
-        iterate(it, std::integral_constant<int, 0>{});
-        if (it + 1 < n_it) iterate(it + 1, std::integral_constant<int, 1>{});
-        if (it + 2 < n_it) iterate(it + 2, std::integral_constant<int, 2>{});
+    // Main pass, unrolled by LDS stage so that every fragment address is (per-lane offset
+    // register) + (immediate).  With kFreeze the first tile runs the exact step and sets every
+    // lane's reference, the others keep it frozen.
+    reset();
+    if constexpr (kFreeze) {
+        if (n_it > 0) {
+            arrive(0);
+            tile_step(0, smem_base, std::true_type{});
+        }
+        for (int it = 1; it < n_it; it += NS) {
+            lean_step(it, std::integral_constant<int, 1>{});
+            if (it + 1 < n_it) lean_step(it + 1, std::integral_constant<int, 2>{});
+            if (it + 2 < n_it) lean_step(it + 2, std::integral_constant<int, 0>{});
+        }
+    } else {
+        for (int it = 0; it < n_it; it += NS) {
+            lean_step(it, std::integral_constant<int, 0>{});
+            if (it + 1 < n_it) lean_step(it + 1, std::integral_constant<int, 1>{});
+            if (it + 2 < n_it) lean_step(it + 2, std::integral_constant<int, 2>{});
+        }
+    }
+    // A sum beyond 2^96 (or not finite) means some logit stood some 95 or more above its row's
+    // reference and the products may have overflowed: the workgroup repeats its key loop with the
+    // exact step on every tile (rare, so this pass has one loop body with a run-time LDS stage).
+    bool unsafe = false;
+#pragma unroll
+    for (int qb = 0; qb < NQB; ++qb) unsafe = unsafe || !(l[qb] < 0x1p96f);
+    if (kFreeze && __syncthreads_or(unsafe)) {
+        reset();
+        int stage = 0;
+        for (int it = 0; it < n_it; ++it) {
+            arrive(it);
+            tile_step(it, smem_base + stage * (2 * kStageTileBytes), std::true_type{});
+            stage = stage == NS - 1 ? 0 : stage + 1;
+        }
     }
 
     // epilogue: z = l + exp(sink - m); O = acc / z; M = m + log z   (ref :93-98)

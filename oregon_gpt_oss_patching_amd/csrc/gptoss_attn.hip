@@ -30,6 +30,12 @@ int check_tensor(const void *p, const gptoss_attn_strides &s, int elem_bytes, in
 
 Strides cvt(const gptoss_attn_strides &s) { return Strides{s.b, s.h, s.s}; }
 
+// A window that reaches back past the first key from every query position is no window: such a
+// call is the full-causal layer and takes exactly its kernels (same bits).
+int effective_window(const gptoss_attn_params *p) {
+    return (p->window > 0 && (int64_t)p->window >= (int64_t)p->Sq + p->q_offset) ? 0 : p->window;
+}
+
 KArgs make_args(const gptoss_attn_params *p) {
     KArgs a{};
     a.q = static_cast<const bf16 *>(p->q);
@@ -50,7 +56,7 @@ KArgs make_args(const gptoss_attn_params *p) {
     a.dos = cvt(p->do_stride); a.dqs = cvt(p->dq_stride); a.dks = cvt(p->dk_stride); a.dvs = cvt(p->dv_stride);
     a.B = p->B; a.H = p->H; a.G = p->G; a.Sq = p->Sq; a.Skv = p->Skv;
     a.r = p->H / p->G;
-    a.window = p->window;
+    a.window = effective_window(p);
     a.q_offset = p->q_offset;
     a.scale = p->scale;
     a.scale_log2 = p->scale * kLog2e;
@@ -82,7 +88,8 @@ int dkdv_parts_for(const gptoss_attn_params *p) {
     if (p->dtype != GPTOSS_ATTN_BF16) return 1;
     const int64_t blocks = (int64_t)p->G * p->B * ((p->Skv + kDkdvKeys - 1) / kDkdvKeys);
     int parts = (int)(1024 / (blocks > 0 ? blocks : 1));
-    const int64_t rows_seen = p->window > 0 ? (int64_t)kDkdvKeys + p->window - 1 : (int64_t)p->Sq;
+    const int window = effective_window(p);
+    const int64_t rows_seen = window > 0 ? (int64_t)kDkdvKeys + window - 1 : (int64_t)p->Sq;
     const int tiles = (int)((rows_seen < p->Sq ? rows_seen : p->Sq) + 63) / 64;
     if (parts > tiles / 4) parts = tiles / 4;
     if (parts > 8) parts = 8;
@@ -109,7 +116,8 @@ int launch(Kernel kernel, int64_t workgroups, int threads, hipStream_t st, const
 // 128 and 2..64 query heads per KV head; everything else keeps the dK/dV + dQ kernel pair.
 bool window_single_pass(const gptoss_attn_params *p) {
     const int r = p->G > 0 ? p->H / p->G : 0;
-    return p->dtype == GPTOSS_ATTN_BF16 && p->window > 0 && p->window <= WinCfg::kMaxWindow && !p->doc_start &&
+    const int window = effective_window(p);
+    return p->dtype == GPTOSS_ATTN_BF16 && window > 0 && window <= WinCfg::kMaxWindow && !p->doc_start &&
            p->q_offset == 0 && p->Sq == p->Skv && r >= 2 && r <= WinCfg::kMaxGroup;
 }
 
