@@ -223,6 +223,32 @@ def test_custom_ops_are_registered_and_match_the_direct_calls():
                           test_utils=("test_schema", "test_faketensor"))
 
 
+@pytest.mark.parametrize("window", [None, 128])
+def test_torch_compile_traces_the_custom_ops(window):
+    """torch.compile (dynamo + AOT autograd, backend "aot_eager", fullgraph) over attention(): the two
+    library calls are opaque custom operators with shape-only implementations, so the traced
+    program calls them unchanged and forward and gradients have the bits of the eager call."""
+    import oregon_gpt_oss_patching_amd as A
+    q, k, v, sinks, d_out = E.make_inputs(14, 2, 16, 2, 384, 64, torch.bfloat16)
+    d_out = d_out.to(DEV)
+
+    def fn(q_, k_, v_, s_):
+        return A.attention(q_, k_, v_, s_, SCALE, window, None)
+
+    eager_in = [t.to(DEV).requires_grad_(True) for t in (q, k, v, sinks)]
+    out_e = fn(*eager_in)
+    out_e.backward(d_out)
+    torch._dynamo.reset()
+    compiled = torch.compile(fn, backend="aot_eager", fullgraph=True)
+    comp_in = [t.to(DEV).requires_grad_(True) for t in (q, k, v, sinks)]
+    out_c = compiled(*comp_in)
+    out_c.backward(d_out)
+    torch.cuda.synchronize()
+    assert torch.equal(out_c, out_e)
+    for a, b in zip(comp_in, eager_in):
+        assert torch.equal(a.grad, b.grad)
+
+
 def test_packed_rows_through_the_patched_model():
     """Packed rows (position ids restarting inside a row).  The stock GPT-OSS eager path of this
     transformers version does not pass position ids to its mask builder, so, like the reference,
