@@ -405,7 +405,7 @@ def test_combined_backward_equals_separate_steps(A, b, h, g, s, w, lens, docs):
     gptoss_attn_bwd runs the same kernels (its dQ kernel computes delta and lse*log2e itself, then
     dSinks, dK/dV) every output has the same bits.  Sliding-window layers with a window of at most
     128 and no packed rows take the single-pass kernel instead, which sums dQ over keys and dK/dV
-    over rows in another order: there the two agree to the last bf16 bit or two."""
+    over rows in another order: there the two agree to within two bf16 units in the last place."""
     q, k, v, sinks, d_out = (t.to(DEV) for t in E.make_inputs(900 + s, b, h, g, s, 64, torch.bfloat16))
     doc_start = None
     if docs is not None:
@@ -425,7 +425,7 @@ def test_combined_backward_equals_separate_steps(A, b, h, g, s, w, lens, docs):
         x, y = x.float(), y.float()
         assert rel_l2(x, y) <= 1e-4, (name, rel_l2(x, y))
         if name != "dsinks":
-            assert bool(((x - y).abs() <= 2.0 ** -7 * torch.maximum(x.abs(), y.abs()) + 1e-6).all()), name
+            assert bool(((x - y).abs() <= 2.0 ** -6 * torch.maximum(x.abs(), y.abs()) + 1e-6).all()), name
 
 
 def test_window_ge_seq_equals_full(A):
