@@ -20,11 +20,18 @@
 //     key tiles resident in its registers) and writes the finished dQ rows.  It also sums the
 //     dSinks terms exp(sink - lse) * (-delta) of its rows.
 // All 192 keys a query tile can see are in the workgroup at the same time, so dQ is complete
-// when the helper stores it.  dK / dV of the chunk's own key tiles [t0, t1) are complete once the
-// walk has gone two query tiles past the chunk (tiles t1, t1+1 are walked for their sake only);
-// the two key tiles before the chunk are walked for the sake of dQ only and their dK / dV are
-// dropped: the neighbouring chunk produces them.  That recomputation replaces any exchange of
-// partial sums between workgroups.
+// when the helper stores it.  A key tile collects from three query tiles, so the last two key
+// tiles of a chunk (and the two before it, which the chunk walks for the sake of its first rows'
+// dQ) are completed by two neighbouring workgroups.  Two ways of closing that seam:
+//   * boundary_partial set (gptoss_attn_bwd): each of the two workgroups leaves its fp32 share of
+//     dK / dV of those tiles in the scratch, and attn_bwd_window_finish_kernel adds the two shares
+//     in a fixed order, scales and rounds: 64 KB of partial sums per seam and tile pair, and a
+//     walk of exactly the chunk's own query tiles;
+//   * boundary_partial NULL (gptoss_attn_bwd_static, which has no room for the partial sums): the
+//     walk goes two query tiles past the chunk, for the sake of its last two key tiles only, and
+//     drops the dK / dV of the two key tiles before the chunk (the neighbour produces them the
+//     same way): recomputation instead of an exchange, 25 % more iterations at 8 tiles per chunk.
+// Both are free of atomics and bit-reproducible.
 //
 // One barrier per iteration hands over the staged Q / dO tile (asynchronous global->LDS copies,
 // three stages), the row statistics of the next tile and the dS tile of the previous one (double
@@ -82,7 +89,8 @@ __global__ __launch_bounds__(WinCfg::NWAVES * 64, 1) void attn_bwd_window_kernel
     const int nT = (a.Sq + kTile - 1) / kTile;
     const int t0 = chunk * a.chunk_tiles;                  // first query tile (and first own key tile)
     const int t1 = min(t0 + a.chunk_tiles, nT);            // end of the chunk
-    const int t_end = min(t1 + 2, nT);                     // two more query tiles complete the chunk's dK / dV
+    const bool seam_sums = a.boundary_partial != nullptr;  // see the file comment
+    const int t_end = seam_sums ? t1 : min(t1 + 2, nT);    // without them two more query tiles complete the chunk's dK / dV
     const int n_it = (t_end - t0) * a.r;
 
     const int kv_len = a.seqlens ? min(a.Skv, a.seqlens[b]) : a.Skv;
@@ -282,8 +290,36 @@ __global__ __launch_bounds__(WinCfg::NWAVES * 64, 1) void attn_bwd_window_kernel
         clear_acc();
     }
     // dK / dV of the key tile held, if it is one of the chunk's own
+    // fp32 share of a seam tile: [b][g][seam][tile 0/1][workgroup before / after the seam][dK, dV][64 keys][64]
+    auto seam_slot = [&](int seam, int tile, int side) {
+        return a.boundary_partial + (((((int64_t)b * a.G + g) * (n_chunks - 1) + seam) * 2 + tile) * 2 + side) * (2 * kTile * kD);
+    };
+    auto store_share = [&](float *dst) {
+        // unscaled fp32 sums; lane = key row, register i of block dblk = column 32*dblk + crow(i, half),
+        // four consecutive columns per 16-byte store
+        float *pk = dst + (32 * sub + l32) * kD, *pv = pk + kTile * kD;
+#pragma unroll
+        for (int dblk = 0; dblk < 2; ++dblk)
+#pragma unroll
+            for (int a4 = 0; a4 < 4; ++a4) {
+                const int col = 32 * dblk + 8 * a4 + 4 * half;
+                f32x4 xk, xv;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) { xk[e] = dk[0][dblk][4 * a4 + e]; xv[e] = dv[0][dblk][4 * a4 + e]; }
+                *reinterpret_cast<f32x4 *>(pk + col) = xk;
+                *reinterpret_cast<f32x4 *>(pv + col) = xv;
+            }
+    };
+    // dK / dV of the key tile held: written out if it is complete, left as this workgroup's share if
+    // it sits on a seam, dropped if it belongs to the neighbour (recomputation mode)
     auto flush = [&]() {
-        if (my_kt < t0 || my_kt >= t1) return;
+        if (my_kt < 0) return;
+        if (seam_sums) {
+            if (my_kt < t0) { store_share(seam_slot(chunk - 1, my_kt - (t0 - 2), 1)); return; }
+            if (my_kt >= t1 - 2 && t1 < nT) { store_share(seam_slot(chunk, my_kt - (t1 - 2), 0)); return; }
+        } else if (my_kt < t0 || my_kt >= t1) {
+            return;
+        }
         const int r0 = my_kt * kTile + 32 * sub;
         const int nvalid = a.Skv - r0;
         store_rows32(out_stage, dk[0], a.scale, a.dk + (int64_t)b * a.dks.b + (int64_t)g * a.dks.h + (int64_t)r0 * a.dks.s,
@@ -421,15 +457,57 @@ __global__ __launch_bounds__(WinCfg::NWAVES * 64, 1) void attn_bwd_window_kernel
 }
 
 // ---------------------------------------------------------------------------------
-// dsinks[h] = sum of the per-(batch, chunk, helper) partial sums the window kernel left, in a
-// fixed order.  One thread per query head.
-__global__ __launch_bounds__(64) void attn_bwd_window_dsinks_kernel(const KArgs a, int n_chunks) {
-    const int h = blockIdx.x * 64 + threadIdx.x;
-    if (h >= a.H) return;
-    float acc = 0.0f;
-    for (int bc = 0; bc < a.B * n_chunks; ++bc)
-        for (int e = 0; e < WinCfg::NHELP; ++e) acc += a.dsink_partial[((int64_t)bc * a.H + h) * WinCfg::NHELP + e];
-    a.dsinks[h] = acc;
+// What is left after the window kernel, in one small launch.  Blocks [0, seam_blocks): dK / dV of
+// the seam tiles = round(scale * (share of the workgroup before the seam + share of the one after)),
+// one thread per 16-byte output chunk.  Blocks from seam_blocks on: one block per query head adds
+// that head's dSinks partial sums (per batch row, chunk and helper) in a fixed tree order.
+__global__ __launch_bounds__(256) void attn_bwd_window_finish_kernel(const KArgs a, int n_chunks, int seam_blocks) {
+    if ((int)blockIdx.x >= seam_blocks) {
+        __shared__ float red[256];
+        const int h = blockIdx.x - seam_blocks;
+        const int n = a.B * n_chunks * WinCfg::NHELP;
+        float acc = 0.0f;
+        for (int i = threadIdx.x; i < n; i += 256) {
+            const int bc = i / WinCfg::NHELP, e = i % WinCfg::NHELP;
+            acc += a.dsink_partial[((int64_t)bc * a.H + h) * WinCfg::NHELP + e];
+        }
+        red[threadIdx.x] = acc;
+        __syncthreads();
+        for (int off = 128; off > 0; off >>= 1) {
+            if ((int)threadIdx.x < off) red[threadIdx.x] += red[threadIdx.x + off];
+            __syncthreads();
+        }
+        if (threadIdx.x == 0) a.dsinks[h] = red[0];
+        return;
+    }
+    // chunk index over (b, g, seam, tile, tensor, key, 8 columns)
+    const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int c8 = (int)(idx & 7) * 8;
+    const int key = (int)((idx >> 3) & 63);
+    const int which = (int)((idx >> 9) & 1);                      // 0 = dK, 1 = dV
+    const int tile = (int)((idx >> 10) & 1);
+    const int64_t rest = idx >> 11;                               // (b * G + g) * (n_chunks - 1) + seam
+    if (rest >= (int64_t)a.B * a.G * (n_chunks - 1)) return;
+    const int seam = (int)(rest % (n_chunks - 1));
+    const int bg = (int)(rest / (n_chunks - 1));
+    const int g = bg % a.G, b = bg / a.G;
+    const int row = ((seam + 1) * a.chunk_tiles - 2 + tile) * kTile + key;
+    if (row >= a.Skv) return;
+    const float *before = a.boundary_partial + ((rest * 2 + tile) * 2 + 0) * (2 * kTile * kD) + (which * kTile + key) * kD + c8;
+    const float *after = before + 2 * kTile * kD;
+    const float mul = which == 0 ? a.scale : 1.0f;
+    bf16x8 out;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const f32x4 x = *reinterpret_cast<const f32x4 *>(before + 4 * j), y = *reinterpret_cast<const f32x4 *>(after + 4 * j);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) out[4 * j + e] = (bf16)((x[e] + y[e]) * mul);
+    }
+    const Strides &st = which == 0 ? a.dks : a.dvs;
+    bf16 *dst = (which == 0 ? a.dk : a.dv) + (int64_t)b * st.b + (int64_t)g * st.h + (int64_t)row * st.s + c8;
+    union { bf16x8 v; u32x4 u; } cv;
+    cv.v = out;
+    *reinterpret_cast<u32x4 *>(dst) = cv.u;
 }
 
 }  // namespace gptoss

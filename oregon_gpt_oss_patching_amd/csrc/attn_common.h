@@ -55,6 +55,7 @@ struct KArgs {
     float *dkdv_partial; // dkdv_parts > 1: fp32 partial sums, [part][dK, dV][B][G][Skv][64]
     int chunk_tiles;     // single-pass window backward: 64-row query tiles per workgroup
     float *dsink_partial; // single-pass window backward: dSinks partial sums, [B][chunk][H][2]
+    float *boundary_partial; // single-pass window backward: fp32 dK / dV shares of the tiles on chunk seams, or NULL
 };
 
 __device__ __forceinline__ int crow(int i, int half) { return 8 * (i >> 2) + 4 * half + (i & 3); }

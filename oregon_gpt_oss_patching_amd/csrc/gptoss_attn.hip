@@ -63,6 +63,7 @@ KArgs make_args(const gptoss_attn_params *p) {
     a.dkdv_parts = 1;
     a.chunk_tiles = 0;
     a.dsink_partial = nullptr;
+    a.boundary_partial = nullptr;
     return a;
 }
 
@@ -160,19 +161,42 @@ int window_lds_attribute() {
     return GPTOSS_ATTN_OK;
 }
 
-int launch_window_bwd(const gptoss_attn_params *p, hipStream_t st) {
+// Scratch of the single-pass window backward: dSinks partial sums [B][chunk][H][2], then (rounded up
+// to 16 bytes) the fp32 dK / dV shares of the two key tiles on each seam between chunks.
+struct WindowScratch { int chunk_tiles, n_chunks; size_t sink_bytes, seam_bytes; };
+
+WindowScratch window_scratch(const gptoss_attn_params *p, int cus) {
+    WindowScratch w;
+    w.chunk_tiles = window_chunk_tiles(p, cus);
+    const int n_tiles = (p->Sq + kTile - 1) / kTile;
+    w.n_chunks = (n_tiles + w.chunk_tiles - 1) / w.chunk_tiles;
+    w.sink_bytes = (((size_t)p->B * w.n_chunks * p->H * WinCfg::NHELP * sizeof(float)) + 15) & ~(size_t)15;
+    w.seam_bytes = (size_t)p->B * p->G * (w.n_chunks - 1) * 2 * 2 * (2 * kTile * kD) * sizeof(float);
+    return w;
+}
+
+// seam_sums: neighbouring chunks exchange fp32 shares through the scratch (needs window_scratch bytes);
+// otherwise each chunk walks two query tiles past its end and nothing but the dSinks sums is kept.
+int launch_window_bwd(const gptoss_attn_params *p, hipStream_t st, bool seam_sums) {
     int rc = window_lds_attribute();
     if (rc) return rc;
     KArgs a = make_args(p);
-    a.chunk_tiles = window_chunk_tiles(p, compute_units());
-    a.dsink_partial = p->delta;                       // the row-statistics part of the scratch is free in this path
-    const int n_tiles = (a.Sq + kTile - 1) / kTile;
-    const int n_chunks = (n_tiles + a.chunk_tiles - 1) / a.chunk_tiles;
-    rc = launch(attn_bwd_window_kernel, (int64_t)a.G * a.B * n_chunks, 64 * WinCfg::NWAVES, st, a, WinCfg::kLdsBytes);
-    if (rc || !a.dsinks) return rc;
-    void *args[] = {&a, const_cast<int *>(&n_chunks)};
-    const hipError_t e = hipLaunchKernel(reinterpret_cast<const void *>(attn_bwd_window_dsinks_kernel), dim3((unsigned)((a.H + 63) / 64)),
-                                         dim3(64), args, 0, st);
+    const WindowScratch ws = window_scratch(p, compute_units());
+    a.chunk_tiles = ws.chunk_tiles;
+    a.dsink_partial = p->delta;
+    if (seam_sums && ws.n_chunks > 1)
+        a.boundary_partial = reinterpret_cast<float *>(reinterpret_cast<char *>(p->delta) + ws.sink_bytes);
+    rc = launch(attn_bwd_window_kernel, (int64_t)a.G * a.B * ws.n_chunks, 64 * WinCfg::NWAVES, st, a, WinCfg::kLdsBytes);
+    if (rc) return rc;
+    // seam tiles and dSinks in one small launch
+    const int64_t seam_chunks = a.boundary_partial ? (int64_t)a.B * a.G * (ws.n_chunks - 1) * 2 * 2 * kTile * 8 : 0;
+    const int seam_blocks = (int)((seam_chunks + 255) / 256);
+    const int sink_blocks = a.dsinks ? a.H : 0;
+    if (seam_blocks + sink_blocks == 0) return GPTOSS_ATTN_OK;
+    int n_chunks = ws.n_chunks, sb = seam_blocks;
+    void *args[] = {&a, &n_chunks, &sb};
+    const hipError_t e = hipLaunchKernel(reinterpret_cast<const void *>(attn_bwd_window_finish_kernel),
+                                         dim3((unsigned)(seam_blocks + sink_blocks)), dim3(256), args, 0, st);
     return e == hipSuccess ? GPTOSS_ATTN_OK : static_cast<int>(e);
 }
 
@@ -247,6 +271,11 @@ size_t gptoss_attn_workspace_bytes(const gptoss_attn_params *p) {
     if (p->G > 0 && p->Skv > 0) {
         const int parts = dkdv_parts_for(p);
         if (parts > 1) n += (size_t)parts * 2 * sizeof(float) * (size_t)p->B * (size_t)p->G * (size_t)p->Skv * kD;
+        if (window_single_pass(p)) {
+            // gptoss_attn_bwd takes this route and lays its own scratch over the same bytes
+            const WindowScratch ws = window_scratch(p, compute_units());
+            if (ws.sink_bytes + ws.seam_bytes > n) n = ws.sink_bytes + ws.seam_bytes;
+        }
     }
     return n;
 }
@@ -331,7 +360,7 @@ static int bwd_all(const gptoss_attn_params *p, void *stream, bool whole_blocks)
         if (rc) return rc;
         return gptoss_attn_bwd_dq(p, stream);
     }
-    if (window_single_pass(p)) return launch_window_bwd(p, static_cast<hipStream_t>(stream));
+    if (window_single_pass(p)) return launch_window_bwd(p, static_cast<hipStream_t>(stream), !whole_blocks);
     rc = launch_dq(p, stream, 1);
     if (rc) return rc;
     if (p->dsinks) {
