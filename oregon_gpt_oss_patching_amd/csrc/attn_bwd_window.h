@@ -77,7 +77,8 @@ __global__ __launch_bounds__(WinCfg::NWAVES * 64, 1) void attn_bwd_window_kernel
     char *const transit = lds + C::kTransitOff;
     float *const ssink = reinterpret_cast<float *>(lds + C::kSinkOff);
 
-    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);   // wave-uniform: keeps everything derived from it in scalar registers
     const int l32 = lane & 31, half = lane >> 5;
     const bool owner = w < C::NOWN;
 

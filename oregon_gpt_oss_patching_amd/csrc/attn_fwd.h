@@ -227,8 +227,10 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_fwd_kernel(const
     const int t_hi = hi > 0 ? (hi + kTile - 1) / kTile : 0;
 
     // this wavefront's own row range (absolute positions)
-    const int wpos0 = a.q_offset + qw0;
-    const int wpos1 = min(a.q_offset + min(a.Sq, qw0 + WM) - 1, q_len - 1);
+    // (wave-uniform values, said so to the compiler: the tile classification below then branches
+    // on scalar conditions)
+    const int wpos0 = __builtin_amdgcn_readfirstlane(a.q_offset + qw0);
+    const int wpos1 = __builtin_amdgcn_readfirstlane(min(a.q_offset + min(a.Sq, qw0 + WM) - 1, q_len - 1));
 
     const bf16 *kbase = a.k + (int64_t)b * a.ks.b + (int64_t)g * a.ks.h;
     const bf16 *vbase = a.v + (int64_t)b * a.vs.b + (int64_t)g * a.vs.h;
