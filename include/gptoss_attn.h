@@ -52,7 +52,7 @@
 extern "C" {
 #endif
 
-#define GPTOSS_ATTN_ABI_VERSION 3
+#define GPTOSS_ATTN_ABI_VERSION 4
 
 enum gptoss_attn_dtype {
     GPTOSS_ATTN_BF16 = 0, /* 2-byte bfloat16 tensors, bf16 MFMA products, fp32 accumulation: the fast path */
@@ -110,6 +110,16 @@ typedef struct gptoss_attn_params {
 
     gptoss_attn_strides q_stride, k_stride, v_stride, o_stride;
     gptoss_attn_strides do_stride, dq_stride, dk_stride, dv_stride;
+
+    /* Optional: device address of one int32 holding the absolute position of query row 0.  When set,
+     * q_offset above is ignored and the kernels read the value themselves (one scalar load per
+     * workgroup), so a caller whose start position lives on the device (the reference reads its
+     * `start_q` tensor inside the kernels, attention_kernel.py:44-47,145-147) neither synchronises
+     * nor bakes the value into a captured graph.  The value must satisfy 0 <= value and
+     * Sq + value <= 2^30 (the kernels clamp it into that range); the host cannot see it, so a window
+     * that covers the whole row is not recognised as full causal, the single-pass window backward
+     * is not taken, and doc_start is refused (ERR_SHAPE). */
+    const int32_t *q_offset_dev;
 } gptoss_attn_params;
 
 /* Library/ABI version (GPTOSS_ATTN_ABI_VERSION it was built with). */

@@ -12,7 +12,7 @@ from typing import Optional
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIBRARY = os.path.join(_HERE, "libgptoss_attn.so")
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 DTYPE_BF16 = 0
 DTYPE_FP32 = 1
 
@@ -59,6 +59,7 @@ class Params(ctypes.Structure):
         ("delta", ctypes.c_void_p),
         ("q_stride", Strides), ("k_stride", Strides), ("v_stride", Strides), ("o_stride", Strides),
         ("do_stride", Strides), ("dq_stride", Strides), ("dk_stride", Strides), ("dv_stride", Strides),
+        ("q_offset_dev", ctypes.c_void_p),
     ]
 
 

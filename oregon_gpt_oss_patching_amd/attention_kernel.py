@@ -104,7 +104,7 @@ def _check_saved(q, o, lse, d_o):
         raise RuntimeError(f"lse must be (B, H, S) = {(b, h, sq)}, got {tuple(lse.shape)}")
 
 
-def _base_params(q, k, v, sinks32, seqlens, scale, window, q_offset, doc_start=None):
+def _base_params(q, k, v, sinks32, seqlens, scale, window, q_offset, doc_start=None, q_offset_dev=None):
     p = _lib.new_params()
     b, h, sq, d = q.shape
     g, skv = k.shape[1], k.shape[2]
@@ -117,6 +117,7 @@ def _base_params(q, k, v, sinks32, seqlens, scale, window, q_offset, doc_start=N
     p.sinks = sinks32.data_ptr() if sinks32 is not None else None
     p.seqlens = seqlens.data_ptr() if seqlens is not None else None
     p.doc_start = doc_start.data_ptr() if doc_start is not None else None
+    p.q_offset_dev = q_offset_dev.data_ptr() if q_offset_dev is not None else None
     _set(p.q_stride, _strides_bhs(q, "bhsd"))
     _set(p.k_stride, _strides_bhs(k, "bhsd"))
     _set(p.v_stride, _strides_bhs(v, "bhsd"))
@@ -134,6 +135,16 @@ def _prep_seqlens(seqlens, device, batch):
     if sl.numel() != batch:
         raise RuntimeError("seqlens must hold one length per batch row")
     return sl
+
+
+def _prep_q_offset_dev(q_offset_dev, q):
+    """One int32 on q's device holding the position of query row 0, or None.  No host read."""
+    if q_offset_dev is None:
+        return None
+    t = q_offset_dev
+    if not torch.is_tensor(t) or t.device != q.device or t.numel() != 1 or t.dtype.is_floating_point:
+        raise RuntimeError("q_offset_dev must be a one-element integer tensor on the same device as q")
+    return t.reshape(1).to(torch.int32).contiguous()
 
 
 def _prep_doc_start(doc_start, q):
@@ -158,18 +169,22 @@ def doc_start_from_position_ids(position_ids: torch.Tensor) -> torch.Tensor:
     return torch.cummax(starts, dim=1).values.to(torch.int32)
 
 
-def attention_forward(q, k, v, sinks, sm_scale, window=None, q_offset=0, seqlens=None, doc_start=None):
-    """Runs the forward kernel.  Returns (o (B,S,H,D), lse (B,H,S) fp32)."""
+def attention_forward(q, k, v, sinks, sm_scale, window=None, q_offset=0, seqlens=None, doc_start=None,
+                      q_offset_dev=None):
+    """Runs the forward kernel.  Returns (o (B,S,H,D), lse (B,H,S) fp32).
+    q_offset_dev: optional one-element integer tensor on the device that holds the query offset
+    (the reference's `start_q` tensor); the kernels read it, the host never does."""
     _check_inputs(q, k, v, sinks)
     q, k, v = _row_contiguous(q), _row_contiguous(k), _row_contiguous(v)
     b, h, sq, d = q.shape
     sinks32 = None if sinks is None else sinks.detach().to(torch.float32).contiguous()
     sl = _prep_seqlens(seqlens, q.device, b)
     ds = _prep_doc_start(doc_start, q)
+    qod = _prep_q_offset_dev(q_offset_dev, q)
     o = torch.empty((b, sq, h, d), dtype=q.dtype, device=q.device)
     lse = torch.empty((b, h, sq), dtype=torch.float32, device=q.device)
     with torch.cuda.device(q.device):
-        p = _base_params(q, k, v, sinks32, sl, sm_scale, window, q_offset, ds)
+        p = _base_params(q, k, v, sinks32, sl, sm_scale, window, q_offset, ds, qod)
         p.o, p.lse = o.data_ptr(), lse.data_ptr()
         _set(p.o_stride, _strides_bhs(o, "bshd"))
         _lib.call("gptoss_attn_fwd", p, _stream(q))
@@ -177,7 +192,7 @@ def attention_forward(q, k, v, sinks, sm_scale, window=None, q_offset=0, seqlens
 
 
 def attention_backward(q, k, v, sinks, o, lse, d_o, sm_scale, window=None, q_offset=0, seqlens=None,
-                       need_dsinks=True, doc_start=None, split=False):
+                       need_dsinks=True, doc_start=None, split=False, q_offset_dev=None):
     """Runs the backward: `gptoss_attn_bwd`, or with `split=True` the three separate entry points
     (preprocess, dK/dV, dQ), which give the same bits.  o and d_o are (B,S,H,D).
     Returns (dq, dk, dv, dsinks_fp32_or_None)."""
@@ -190,12 +205,13 @@ def attention_backward(q, k, v, sinks, o, lse, d_o, sm_scale, window=None, q_off
     sinks32 = None if sinks is None else sinks.detach().to(torch.float32).contiguous()
     sl = _prep_seqlens(seqlens, q.device, b)
     ds = _prep_doc_start(doc_start, q)
+    qod = _prep_q_offset_dev(q_offset_dev, q)
     dq = torch.empty((b, h, sq, d), dtype=q.dtype, device=q.device)
     dk = torch.empty(k.shape, dtype=k.dtype, device=q.device)
     dv = torch.empty(v.shape, dtype=v.dtype, device=q.device)
     dsinks = torch.empty((h,), dtype=torch.float32, device=q.device) if need_dsinks else None
     with torch.cuda.device(q.device):
-        p = _base_params(q, k, v, sinks32, sl, sm_scale, window, q_offset, ds)
+        p = _base_params(q, k, v, sinks32, sl, sm_scale, window, q_offset, ds, qod)
         # scratch: [-delta; lse*log2e], then the dK/dV partial sums of split key blocks (short sequences)
         delta = torch.empty((_lib.load().gptoss_attn_workspace_bytes(p) // 4,), dtype=torch.float32, device=q.device)
         p.o, p.lse = o.data_ptr(), lse.data_ptr()
@@ -225,12 +241,13 @@ OP_NAMESPACE = "gptoss_attn"
 @torch.library.custom_op(f"{OP_NAMESPACE}::fwd", mutates_args=(), device_types="cuda")
 def _op_fwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, sinks: Optional[torch.Tensor], sm_scale: float,
             window: int, q_offset: int, seqlens: Optional[torch.Tensor],
-            doc_start: Optional[torch.Tensor]) -> Tuple[torch.Tensor, torch.Tensor]:
-    return attention_forward(q, k, v, sinks, sm_scale, window, q_offset, seqlens, doc_start)
+            doc_start: Optional[torch.Tensor],
+            q_offset_dev: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
+    return attention_forward(q, k, v, sinks, sm_scale, window, q_offset, seqlens, doc_start, q_offset_dev)
 
 
 @_op_fwd.register_fake
-def _op_fwd_fake(q, k, v, sinks, sm_scale, window, q_offset, seqlens, doc_start):
+def _op_fwd_fake(q, k, v, sinks, sm_scale, window, q_offset, seqlens, doc_start, q_offset_dev=None):
     b, h, sq, d = q.shape
     return q.new_empty((b, sq, h, d)), q.new_empty((b, h, sq), dtype=torch.float32)
 
@@ -239,16 +256,18 @@ def _op_fwd_fake(q, k, v, sinks, sm_scale, window, q_offset, seqlens, doc_start)
 def _op_bwd(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, sinks: Optional[torch.Tensor], o: torch.Tensor,
             lse: torch.Tensor, d_o: torch.Tensor, sm_scale: float, window: int, q_offset: int,
             seqlens: Optional[torch.Tensor], doc_start: Optional[torch.Tensor],
-            need_dsinks: bool) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
+            need_dsinks: bool,
+            q_offset_dev: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, torch.Tensor]:
     dq, dk, dv, dsinks = attention_backward(q, k, v, sinks, o, lse, d_o, sm_scale, window, q_offset, seqlens,
-                                            need_dsinks=need_dsinks, doc_start=doc_start)
+                                            need_dsinks=need_dsinks, doc_start=doc_start, q_offset_dev=q_offset_dev)
     if dsinks is None:      # an operator cannot return None: an empty tensor stands for "not requested"
         dsinks = torch.empty((0,), dtype=torch.float32, device=q.device)
     return dq, dk, dv, dsinks
 
 
 @_op_bwd.register_fake
-def _op_bwd_fake(q, k, v, sinks, o, lse, d_o, sm_scale, window, q_offset, seqlens, doc_start, need_dsinks):
+def _op_bwd_fake(q, k, v, sinks, o, lse, d_o, sm_scale, window, q_offset, seqlens, doc_start, need_dsinks,
+                 q_offset_dev=None):
     return (torch.empty_like(q, memory_format=torch.contiguous_format),
             torch.empty_like(k, memory_format=torch.contiguous_format),
             torch.empty_like(v, memory_format=torch.contiguous_format),
@@ -269,15 +288,19 @@ class _attention(torch.autograd.Function):
         ctx.in_dtypes = (q.dtype, k.dtype, v.dtype)
         if q.dtype == torch.float16:
             q, k, v = (t.to(torch.bfloat16) for t in (q, k, v))
-        q_offset = 0
-        if start_q is not None:
+        # a start_q tensor that lives on the device stays there: the kernels read it (as the
+        # reference's do, attention_kernel.py:44-47), the host does not wait for it
+        q_offset, q_offset_dev = 0, None
+        if torch.is_tensor(start_q) and start_q.is_cuda:
+            q_offset_dev = _prep_q_offset_dev(start_q, q)
+        elif start_q is not None:
             q_offset = int(start_q.item()) if torch.is_tensor(start_q) else int(start_q)
         seqlens = _prep_seqlens(seqlens, q.device, q.shape[0])
         doc_start = _prep_doc_start(doc_start, q)
         window = int(bandwidth or 0)
         sinks_in = None if sinks is None else sinks.detach()
-        o, lse = _op_fwd(q, k, v, sinks_in, float(sm_scale), window, q_offset, seqlens, doc_start)
-        ctx.save_for_backward(q, k, v, sinks, o, lse, seqlens, doc_start)
+        o, lse = _op_fwd(q, k, v, sinks_in, float(sm_scale), window, q_offset, seqlens, doc_start, q_offset_dev)
+        ctx.save_for_backward(q, k, v, sinks, o, lse, seqlens, doc_start, q_offset_dev)
         ctx.sm_scale = float(sm_scale)
         ctx.window = window
         ctx.q_offset = q_offset
@@ -285,11 +308,11 @@ class _attention(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, do):
-        q, k, v, sinks, o, lse, seqlens, doc_start = ctx.saved_tensors
+        q, k, v, sinks, o, lse, seqlens, doc_start, q_offset_dev = ctx.saved_tensors
         need_ds = sinks is not None and ctx.needs_input_grad[3]
         sinks_in = None if sinks is None else sinks.detach()
         dq, dk, dv, dsinks = _op_bwd(q, k, v, sinks_in, o, lse, do.to(q.dtype), ctx.sm_scale, ctx.window,
-                                     ctx.q_offset, seqlens, doc_start, need_ds)
+                                     ctx.q_offset, seqlens, doc_start, need_ds, q_offset_dev)
         dsinks = dsinks.to(sinks.dtype).view_as(sinks) if need_ds else None
         qd, kd, vd = ctx.in_dtypes
         return dq.to(qd), dk.to(kd), dv.to(vd), dsinks, None, None, None, None, None

@@ -233,6 +233,7 @@ __device__ __forceinline__ void dkdv_tile(uint32_t qsm, uint32_t gsm, uint32_t s
 
 template <int NW, int NB, bool DOCS>  // NB = 32-key blocks per wavefront; DOCS = packed rows (doc_start given)
 __global__ __launch_bounds__(NW * 64, (NB == 1 ? 2 : 1)) void attn_bwd_dkdv_kernel(const KArgs a) {
+    const int q_offset = query_offset(a);
     static_assert(NW == 4, "the asynchronous tile copy is written for 4 wavefronts");
     constexpr int NS = 3;              // LDS stages: tiles are requested two iterations ahead
     constexpr int WK = 32 * NB;        // keys per wavefront
@@ -258,9 +259,9 @@ __global__ __launch_bounds__(NW * 64, (NB == 1 ? 2 : 1)) void attn_bwd_dkdv_kern
 
     // query rows that can see any key of the workgroup
     const int j1 = min(j0 + BN, kv_len) - 1;              // last live key
-    const int i_lo = max(0, j0 - a.q_offset);
-    int64_t i_hi64 = min((int64_t)a.Sq, (int64_t)q_len - a.q_offset);
-    i_hi64 = min(i_hi64, (int64_t)j1 + weff - a.q_offset);
+    const int i_lo = max(0, j0 - q_offset);
+    int64_t i_hi64 = min((int64_t)a.Sq, (int64_t)q_len - q_offset);
+    i_hi64 = min(i_hi64, (int64_t)j1 + weff - q_offset);
     const int i_hi = (j1 >= j0) ? (int)max((int64_t)0, i_hi64) : 0;
     // With dkdv_parts > 1 the query tiles of the key block (walked from the last one down) are cut
     // into dkdv_parts consecutive slices, one per workgroup; each leaves an fp32 partial sum and
@@ -376,12 +377,12 @@ __global__ __launch_bounds__(NW * 64, (NB == 1 ? 2 : 1)) void attn_bwd_dkdv_kern
         const uint32_t ds_lane = doc_base + STAGE * (kTile * 4) + half * 16;
         const int i0 = cur_i0;
         if (++cur_h == a.r) { cur_h = 0; cur_i0 -= kTile; }
-        const int pos0 = a.q_offset + i0;                                    // first query position of the tile
-        const int pos1 = min(a.q_offset + min(a.Sq, i0 + kTile) - 1, q_len - 1);   // last live one
+        const int pos0 = q_offset + i0;                                    // first query position of the tile
+        const int pos1 = min(q_offset + min(a.Sq, i0 + kTile) - 1, q_len - 1);   // last live one
         const int wj1 = min(wj0 + WK, kv_len) - 1;                           // wavefront's last live key
         bool skip = wj1 < wj0 || pos1 < wj0 || pos0 > wj1 + weff - 1 || pos1 < pos0;
         bool interior = (wj0 + WK - 1 <= pos0) && (wj0 > pos1 - weff) && (wj0 + WK <= kv_len) &&
-                        (a.q_offset + i0 + kTile - 1 <= pos1);
+                        (q_offset + i0 + kTile - 1 <= pos1);
         if constexpr (DOCS) {
             // document starts never decrease along a row: the tile's first row has the smallest,
             // its last row the largest (rows past the end repeat the last valid one)
@@ -400,7 +401,7 @@ __global__ __launch_bounds__(NW * 64, (NB == 1 ? 2 : 1)) void attn_bwd_dkdv_kern
                 const int j = wj0 + 32 * nb + l32;
                 dbase[nb] = (j < kv_len) ? pos0 - j : -0x40000000;
             }
-            const int row_lim = (int)min((int64_t)kTile, min((int64_t)a.Sq, (int64_t)q_len - a.q_offset) - i0);
+            const int row_lim = (int)min((int64_t)kTile, min((int64_t)a.Sq, (int64_t)q_len - q_offset) - i0);
             dkdv_tile<true, DOCS, NB>(qsm, gsm, stat_lane, lo, kf, vf, dk, dv, c, half, dbase, (unsigned)weff, row_lim,
                                       wj0 - pos0, ds_lane, jkey);
         }
@@ -552,6 +553,7 @@ __device__ __forceinline__ void dq_tile(uint32_t ksm, uint32_t vsm, const TileLa
 
 template <int HPB, int NQB, bool FUSE_DELTA>   // FUSE_DELTA: also produce the row statistics of the wavefront's own rows
 __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_bwd_dq_kernel(const KArgs a) {
+    const int q_offset = query_offset(a);
     constexpr int QSUB = 4 / HPB;
     constexpr int WM = 32 * NQB;
     constexpr int BM = WM * QSUB;
@@ -578,8 +580,8 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_bwd_dq_kernel(co
     const int q_len = a.seqlens ? a.seqlens[b] : 0x7fffffff;
     const int weff = a.window ? a.window : 0x3fffffff;
 
-    const int bpos0 = a.q_offset + qt * BM;
-    const int bpos1 = min(a.q_offset + min(a.Sq, (qt + 1) * BM) - 1, q_len - 1);
+    const int bpos0 = q_offset + qt * BM;
+    const int bpos1 = min(q_offset + min(a.Sq, (qt + 1) * BM) - 1, q_len - 1);
     const int hi = bpos1 >= bpos0 ? min(kv_len, bpos1 + 1) : 0;
     const int key_lo = max(0, bpos0 - weff + 1);
     const int32_t *dsrow = a.doc_start ? a.doc_start + (int64_t)b * a.Sq : nullptr;
@@ -589,8 +591,8 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_bwd_dq_kernel(co
     const int t_lo = max(key_lo, ds_b0) / kTile;
     const int t_hi = hi > 0 ? (hi + kTile - 1) / kTile : 0;
 
-    const int wpos0 = a.q_offset + qw0;
-    const int wpos1 = min(a.q_offset + min(a.Sq, qw0 + WM) - 1, q_len - 1);
+    const int wpos0 = q_offset + qw0;
+    const int wpos1 = min(q_offset + min(a.Sq, qw0 + WM) - 1, q_len - 1);
 
     const bf16 *kbase = a.k + (int64_t)b * a.ks.b + (int64_t)g * a.ks.h;
     const bf16 *vbase = a.v + (int64_t)b * a.vs.b + (int64_t)g * a.vs.h;
@@ -650,7 +652,7 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_bwd_dq_kernel(co
             lse2[qb] = a.delta[(int64_t)a.B * a.H * a.Sq + off];   // lse * log2(e), written by the delta kernel
             dlt[qb] = a.delta[off];                                  // -delta
         }
-        const int p = a.q_offset + row;
+        const int p = q_offset + row;
         pq[qb] = (row_ok && p < q_len) ? p : -0x40000000;
         wl[qb] = (unsigned)weff;
         if (dsrow && row_ok) wl[qb] = (unsigned)min(weff, p - dsrow[row] + 1);
@@ -699,7 +701,7 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_bwd_dq_kernel(co
                           (n0 + kTile - 1) < ds_w0;
         if (skip) return;
         const bool interior = (n0 + kTile - 1 <= wpos0) && (n0 > wpos1 - weff) && (n0 + kTile <= kv_len) &&
-                              (a.q_offset + qw0 + WM - 1 <= wpos1) && (n0 >= ds_w1);
+                              (q_offset + qw0 + WM - 1 <= wpos1) && (n0 >= ds_w1);
         if (interior) {
             dq_tile<false, NQB>(ksm, vsm, lo, qf, gf, dq, lse2, dlt, dseed, c, lane, pq, wl, 0u, 0, 0);
         } else {

@@ -49,6 +49,7 @@ struct KArgs {
     int r;               // H / G query heads per KV head
     int window;          // 0 = full causal
     int q_offset;
+    const int32_t *q_offset_dev;  // if set, the offset is read from device memory and q_offset is ignored
     float scale;
     float scale_log2;    // scale * log2(e)
     int dkdv_parts;      // dK/dV kernel: workgroups that share one key block, each taking a slice of its query tiles
@@ -57,6 +58,15 @@ struct KArgs {
     float *dsink_partial; // single-pass window backward: dSinks partial sums, [B][chunk][H][2]
     float *boundary_partial; // single-pass window backward: fp32 dK / dV shares of the tiles on chunk seams, or NULL
 };
+
+// Absolute position of query row 0: by value, or (for callers that must not synchronise with the
+// device to learn it) from device memory, one scalar load per workgroup.
+__device__ __forceinline__ int query_offset(const KArgs &a) {
+    if (!a.q_offset_dev) return a.q_offset;
+    const int v = __builtin_amdgcn_readfirstlane(*a.q_offset_dev);
+    return min(max(v, 0), (1 << 30) - a.Sq);      // what the host checks for an offset passed by value
+}
+
 
 __device__ __forceinline__ int crow(int i, int half) { return 8 * (i >> 2) + 4 * half + (i & 3); }
 

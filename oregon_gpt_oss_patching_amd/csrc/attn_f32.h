@@ -59,9 +59,9 @@ struct RowInfo {
     int pos;        // absolute position, hugely negative for a row that does not exist / is padding
     unsigned win;   // visible keys are pos - win < key <= pos
 };
-__device__ __forceinline__ RowInfo row_info(const KArgs &a, int b, int row, int q_len) {
+__device__ __forceinline__ RowInfo row_info(const KArgs &a, int q_offset, int b, int row, int q_len) {
     RowInfo r;
-    const int p = a.q_offset + row;
+    const int p = q_offset + row;
     const bool live = row < a.Sq && p < q_len;
     r.pos = live ? p : -0x40000000;
     int w = a.window ? a.window : 0x3fffffff;
@@ -85,6 +85,7 @@ __device__ __forceinline__ bool wave_work(int n_blk, int n_head, int n_batch, in
 
 // ---- forward ------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void attn_f32_fwd_kernel(const KArgs a) {
+    const int q_offset = query_offset(a);
     const F32Ptrs t = f32_ptrs(a);
     const int lane = threadIdx.x & 63, l32 = lane & 31, half = lane >> 5;
     int b, head, qblk;
@@ -93,7 +94,7 @@ __global__ __launch_bounds__(256) void attn_f32_fwd_kernel(const KArgs a) {
     const int kv_len = a.seqlens ? min(a.Skv, a.seqlens[b]) : a.Skv;
     const int q_len = a.seqlens ? a.seqlens[b] : 0x7fffffff;
     const int q0 = 32 * qblk, row = q0 + l32;
-    const RowInfo ri = row_info(a, b, row, q_len);
+    const RowInfo ri = row_info(a, q_offset, b, row, q_len);
 
     float qr[32];    // Q[row][32*half + ks]
     load_row32(qr, t.q + (int64_t)b * a.qs.b + (int64_t)head * a.qs.h + (int64_t)min(row, a.Sq - 1) * a.qs.s + 32 * half, row < a.Sq);
@@ -109,9 +110,9 @@ __global__ __launch_bounds__(256) void attn_f32_fwd_kernel(const KArgs a) {
 
     // keys any row of this block can see: [key_lo, key_hi)
     const int weff = a.window ? a.window : 0x3fffffff;
-    const int pos_hi = min(a.q_offset + min(a.Sq, q0 + 32) - 1, q_len - 1);
-    const int key_hi = pos_hi >= a.q_offset + q0 ? min(kv_len, pos_hi + 1) : 0;
-    const int key_lo = max(0, a.q_offset + q0 - weff + 1);
+    const int pos_hi = min(q_offset + min(a.Sq, q0 + 32) - 1, q_len - 1);
+    const int key_hi = pos_hi >= q_offset + q0 ? min(kv_len, pos_hi + 1) : 0;
+    const int key_lo = max(0, q_offset + q0 - weff + 1);
     for (int n0 = (key_lo / 32) * 32; n0 < key_hi; n0 += 32) {
         float kr[32];    // K[n0 + l32][32*half + ks]
         load_row32(kr, kb + (int64_t)min(n0 + l32, a.Skv - 1) * a.ks.s + 32 * half, true);
@@ -195,6 +196,7 @@ __global__ __launch_bounds__(256) void attn_f32_delta_kernel(const KArgs a) {
 
 // ---- backward step 2: dK, dV ------------------------------------------------------------
 __global__ __launch_bounds__(256) void attn_f32_dkdv_kernel(const KArgs a) {
+    const int q_offset = query_offset(a);
     const F32Ptrs t = f32_ptrs(a);
     const int lane = threadIdx.x & 63, l32 = lane & 31, half = lane >> 5;
     int b, g, kblk;
@@ -213,8 +215,8 @@ __global__ __launch_bounds__(256) void attn_f32_dkdv_kernel(const KArgs a) {
 
     // query rows that can see any key of the block: positions [j0, j0 + 31 + window)
     const int weff = a.window ? a.window : 0x3fffffff;
-    const int row_lo = max(0, j0 - a.q_offset);
-    const int64_t row_hi64 = min((int64_t)min(a.Sq, max(0, q_len - a.q_offset)), (int64_t)j0 + 31 + weff - a.q_offset);
+    const int row_lo = max(0, j0 - q_offset);
+    const int64_t row_hi64 = min((int64_t)min(a.Sq, max(0, q_len - q_offset)), (int64_t)j0 + 31 + weff - q_offset);
     const int row_hi = j0 < kv_len ? (int)row_hi64 : 0;
     const float c = a.scale_log2;
     for (int hh = 0; hh < a.r; ++hh) {
@@ -242,7 +244,7 @@ __global__ __launch_bounds__(256) void attn_f32_dkdv_kernel(const KArgs a) {
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 const int row = q0 + crow(i, half);
-                RowInfo ri = row_info(a, b, row, q_len);
+                RowInfo ri = row_info(a, q_offset, b, row, q_len);
                 const float p = visible(ri, key, kv_len) ? exp2f(fmaf(s[i], c, -l2[min(row, a.Sq - 1)])) : 0.0f;
                 s[i] = p;
                 dp[i] = p * dp[i];                                        // dS (without the softmax scale)
@@ -281,6 +283,7 @@ __global__ __launch_bounds__(256) void attn_f32_dkdv_kernel(const KArgs a) {
 
 // ---- backward step 3: dQ ----------------------------------------------------------------
 __global__ __launch_bounds__(256) void attn_f32_dq_kernel(const KArgs a) {
+    const int q_offset = query_offset(a);
     const F32Ptrs t = f32_ptrs(a);
     const int lane = threadIdx.x & 63, l32 = lane & 31, half = lane >> 5;
     int b, head, qblk;
@@ -289,7 +292,7 @@ __global__ __launch_bounds__(256) void attn_f32_dq_kernel(const KArgs a) {
     const int kv_len = a.seqlens ? min(a.Skv, a.seqlens[b]) : a.Skv;
     const int q_len = a.seqlens ? a.seqlens[b] : 0x7fffffff;
     const int q0 = 32 * qblk, row = q0 + l32;
-    const RowInfo ri = row_info(a, b, row, q_len);
+    const RowInfo ri = row_info(a, q_offset, b, row, q_len);
     const int64_t total = (int64_t)a.B * a.H * a.Sq;
     const int rowc = min(row, a.Sq - 1);
 
@@ -306,9 +309,9 @@ __global__ __launch_bounds__(256) void attn_f32_dq_kernel(const KArgs a) {
     for (int i = 0; i < 16; ++i) { dq[0][i] = 0.0f; dq[1][i] = 0.0f; }
 
     const int weff = a.window ? a.window : 0x3fffffff;
-    const int pos_hi = min(a.q_offset + min(a.Sq, q0 + 32) - 1, q_len - 1);
-    const int key_hi = pos_hi >= a.q_offset + q0 ? min(kv_len, pos_hi + 1) : 0;
-    const int key_lo = max(0, a.q_offset + q0 - weff + 1);
+    const int pos_hi = min(q_offset + min(a.Sq, q0 + 32) - 1, q_len - 1);
+    const int key_hi = pos_hi >= q_offset + q0 ? min(kv_len, pos_hi + 1) : 0;
+    const int key_lo = max(0, q_offset + q0 - weff + 1);
     for (int n0 = (key_lo / 32) * 32; n0 < key_hi; n0 += 32) {
         const int krow = min(n0 + l32, a.Skv - 1);
         float kr[32], vr[32];

@@ -182,6 +182,7 @@ __device__ __forceinline__ void fwd_tile_lean(uint32_t ksm, uint32_t vsm, const 
 
 template <int HPB, int NQB>
 __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_fwd_kernel(const KArgs a) {
+    const int q_offset = query_offset(a);
     constexpr int QSUB = 4 / HPB;      // row slabs per workgroup
     constexpr int WM = 32 * NQB;       // query rows per wavefront
     constexpr int BM = WM * QSUB;      // query rows per workgroup
@@ -213,8 +214,8 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_fwd_kernel(const
     const int weff = a.window ? a.window : 0x3fffffff;
 
     // key range of the workgroup (union over its wavefronts)
-    const int bpos0 = a.q_offset + qt * BM;
-    const int bpos1 = min(a.q_offset + min(a.Sq, (qt + 1) * BM) - 1, q_len - 1);
+    const int bpos0 = q_offset + qt * BM;
+    const int bpos1 = min(q_offset + min(a.Sq, (qt + 1) * BM) - 1, q_len - 1);
     const int hi = bpos1 >= bpos0 ? min(kv_len, bpos1 + 1) : 0;   // no key at all for a fully padded tile
     const int key_lo = max(0, bpos0 - weff + 1);
     // packed rows: first key of the document of the workgroup's first row (document starts never
@@ -229,8 +230,8 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_fwd_kernel(const
     // this wavefront's own row range (absolute positions)
     // (wave-uniform values, said so to the compiler: the tile classification below then branches
     // on scalar conditions)
-    const int wpos0 = __builtin_amdgcn_readfirstlane(a.q_offset + qw0);
-    const int wpos1 = __builtin_amdgcn_readfirstlane(min(a.q_offset + min(a.Sq, qw0 + WM) - 1, q_len - 1));
+    const int wpos0 = __builtin_amdgcn_readfirstlane(q_offset + qw0);
+    const int wpos1 = __builtin_amdgcn_readfirstlane(min(q_offset + min(a.Sq, qw0 + WM) - 1, q_len - 1));
 
     const bf16 *kbase = a.k + (int64_t)b * a.ks.b + (int64_t)g * a.ks.h;
     const bf16 *vbase = a.v + (int64_t)b * a.vs.b + (int64_t)g * a.vs.h;
@@ -249,7 +250,7 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_fwd_kernel(const
             if (row < a.Sq) z = *reinterpret_cast<const u32x4 *>(qrow + 16 * ks + 8 * half);
             qf[qb][ks] = as_bf16x8(z);
         }
-        const int p = a.q_offset + row;
+        const int p = q_offset + row;
         pq[qb] = (row < a.Sq && p < q_len) ? p : -0x40000000;
         wl[qb] = (unsigned)weff;
         if (dsrow && row < a.Sq) wl[qb] = (unsigned)min(weff, p - dsrow[row] + 1);
@@ -317,7 +318,7 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_fwd_kernel(const
                           (n0 + kTile - 1) < ds_w0;
         if (skip) return;
         const bool interior = (n0 + kTile - 1 <= wpos0) && (n0 > wpos1 - weff) && (n0 + kTile <= kv_len) &&
-                              (a.q_offset + qw0 + WM - 1 <= wpos1) && (n0 >= ds_w1);
+                              (q_offset + qw0 + WM - 1 <= wpos1) && (n0 >= ds_w1);
         int dbase[NQB];
 #pragma unroll
         for (int qb = 0; qb < NQB; ++qb) dbase[qb] = pq[qb] - n0;   // stays hugely negative for dead rows

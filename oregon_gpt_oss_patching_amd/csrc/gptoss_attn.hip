@@ -32,7 +32,9 @@ Strides cvt(const gptoss_attn_strides &s) { return Strides{s.b, s.h, s.s}; }
 
 // A window that reaches back past the first key from every query position is no window: such a
 // call is the full-causal layer and takes exactly its kernels (same bits).
+// (Not decidable on the host when the query offset lives in device memory.)
 int effective_window(const gptoss_attn_params *p) {
+    if (p->q_offset_dev) return p->window;
     return (p->window > 0 && (int64_t)p->window >= (int64_t)p->Sq + p->q_offset) ? 0 : p->window;
 }
 
@@ -57,7 +59,8 @@ KArgs make_args(const gptoss_attn_params *p) {
     a.B = p->B; a.H = p->H; a.G = p->G; a.Sq = p->Sq; a.Skv = p->Skv;
     a.r = p->H / p->G;
     a.window = effective_window(p);
-    a.q_offset = p->q_offset;
+    a.q_offset = p->q_offset_dev ? 0 : p->q_offset;
+    a.q_offset_dev = p->q_offset_dev;
     a.scale = p->scale;
     a.scale_log2 = p->scale * kLog2e;
     a.dkdv_parts = 1;
@@ -119,7 +122,7 @@ bool window_single_pass(const gptoss_attn_params *p) {
     const int r = p->G > 0 ? p->H / p->G : 0;
     const int window = effective_window(p);
     return p->dtype == GPTOSS_ATTN_BF16 && window > 0 && window <= WinCfg::kMaxWindow && !p->doc_start &&
-           p->q_offset == 0 && p->Sq == p->Skv && r >= 2 && r <= WinCfg::kMaxGroup;
+           p->q_offset == 0 && !p->q_offset_dev && p->Sq == p->Skv && r >= 2 && r <= WinCfg::kMaxGroup;
 }
 
 constexpr int kMaxDevices = 64;
@@ -236,11 +239,12 @@ int gptoss_attn_validate(const gptoss_attn_params *p, int need_bwd) {
     if (p->dtype != GPTOSS_ATTN_BF16 && p->dtype != GPTOSS_ATTN_FP32) return GPTOSS_ATTN_ERR_DTYPE;
     if (p->D != kD) return GPTOSS_ATTN_ERR_HEAD_DIM;
     if (p->H <= 0 || p->G <= 0 || p->H % p->G) return GPTOSS_ATTN_ERR_HEADS;
-    if (p->B <= 0 || p->Sq <= 0 || p->Skv <= 0 || p->window < 0 || p->q_offset < 0) return GPTOSS_ATTN_ERR_SHAPE;
+    if (p->B <= 0 || p->Sq <= 0 || p->Skv <= 0 || p->window < 0 || (!p->q_offset_dev && p->q_offset < 0)) return GPTOSS_ATTN_ERR_SHAPE;
     // positions are 32-bit in the kernels and +-2^30 marks "no window" / "dead row"
-    if ((int64_t)p->Sq + p->q_offset > (1 << 30) || p->Skv > (1 << 30) || p->window > (1 << 30)) return GPTOSS_ATTN_ERR_SHAPE;
+    if ((int64_t)p->Sq + (p->q_offset_dev ? 0 : p->q_offset) > (1 << 30) || p->Skv > (1 << 30) || p->window > (1 << 30)) return GPTOSS_ATTN_ERR_SHAPE;
     if (!(p->scale > 0.0f) || !(p->scale < 3.0e38f)) return GPTOSS_ATTN_ERR_SHAPE;
-    if (p->doc_start && (p->Sq != p->Skv || p->q_offset != 0)) return GPTOSS_ATTN_ERR_SHAPE;
+    if (p->doc_start && (p->Sq != p->Skv || p->q_offset != 0 || p->q_offset_dev)) return GPTOSS_ATTN_ERR_SHAPE;
+    if (p->q_offset_dev && (reinterpret_cast<uintptr_t>(p->q_offset_dev) & 3)) return GPTOSS_ATTN_ERR_ALIGNMENT;
     const int eb = p->dtype == GPTOSS_ATTN_FP32 ? 4 : 2;
     int rc;
     if ((rc = check_tensor(p->q, p->q_stride, eb, p->D))) return rc;

@@ -47,7 +47,7 @@ def test_struct_mirror_matches_header_field_order():
         for part in decl.split(","):
             names.append(re.findall(r"[A-Za-z_][A-Za-z_0-9]*", part)[-1])
     assert names == [f[0] for f in _lib.Params._fields_]
-    assert ctypes.sizeof(_lib.Params) == 352
+    assert ctypes.sizeof(_lib.Params) == 360
 
 
 def _valid_params():
@@ -97,12 +97,31 @@ def test_validate_accepts_good_params():
     (lambda p: setattr(p.q_stride, "s", 2 ** 24 + 64), -8),
     (lambda p: (setattr(p, "doc_start", 0x2000), setattr(p, "q_offset", 4)), -5),
     (lambda p: (setattr(p, "doc_start", 0x2000), setattr(p, "Skv", 256)), -5),
+    (lambda p: (setattr(p, "doc_start", 0x2000), setattr(p, "q_offset_dev", 0x3000)), -5),
+    (lambda p: setattr(p, "q_offset_dev", 0x3002), -7),
 ])
 def test_validate_error_codes(mutate, code):
     p = _valid_params()
     mutate(p)
     assert _validate(p) == code
     assert _lib.status_string(code) not in ("ok", "unknown status")
+
+
+def test_device_query_offset_overrides_the_host_field():
+    """With q_offset_dev set the host field is not looked at (the kernels read the device value),
+    and the host-side shortcuts that need the value are off: the workspace is the generic one."""
+    p = _valid_params()
+    p.q_offset_dev = 0x3000
+    p.q_offset = -7
+    assert _validate(p) == 0
+    lib = _lib.load()
+    q = _valid_params()
+    q.window = 128
+    single_pass = lib.gptoss_attn_workspace_bytes(ctypes.byref(q))
+    q.q_offset_dev = 0x3000
+    generic = lib.gptoss_attn_workspace_bytes(ctypes.byref(q))
+    q.q_offset_dev, q.window = None, 0
+    assert generic == lib.gptoss_attn_workspace_bytes(ctypes.byref(q)) and single_pass >= generic
 
 
 def test_forward_only_validation_ignores_backward_tensors():
@@ -161,7 +180,14 @@ def test_workspace_bytes():
     p.B, p.Sq, p.Skv = 1, 4096, 4096
     stats = 2 * 4 * 1 * 64 * 4096
     assert lib.gptoss_attn_workspace_bytes(ctypes.byref(p)) == stats + 4 * 2 * 4 * 1 * 8 * 4096 * 64
+    # a sliding-window layer the single-pass backward takes: its dSinks partial sums [B][chunks][H][2]
+    # and 128 KB of fp32 dK/dV shares per (batch, KV head, seam between chunks), if that is more than
+    # the row statistics.  64 query tiles x 8 KV heads over 256 compute units (the count assumed
+    # without a device, and MI355X's) = 2 tiles per chunk, 32 chunks.
     p.window = 128
+    chunks = 32
+    assert lib.gptoss_attn_workspace_bytes(ctypes.byref(p)) == 1 * chunks * 64 * 2 * 4 + 1 * 8 * (chunks - 1) * 128 * 1024
+    p.window = 256      # longer windows take the three-kernel route: row statistics only, never cut
     assert lib.gptoss_attn_workspace_bytes(ctypes.byref(p)) == stats
     p.window = 0
     p.dtype = _lib.DTYPE_FP32

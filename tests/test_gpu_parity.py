@@ -366,6 +366,35 @@ def test_q_offset_and_longer_kv(A):
         compare_all(run_hip(A, *inp, w, 24), oracle_eager(*inp, w, 24))
 
 
+def test_query_offset_from_device_memory(A):
+    """The offset read by the kernels from device memory (the reference's start_q tensor,
+    attention_kernel.py:44-47) gives the bits of the same offset passed by value; the value passed
+    by value next to it is ignored.  Both dtypes, both layer types, through autograd as well."""
+    for dtype in (torch.bfloat16, torch.float32):
+        for w in (None, 16):
+            q, k, v, sinks, d_out = E.make_inputs(31, 1, 8, 2, 40, 64, dtype, skv=64)
+            qd, kd, vd, sd, dod = (t.to(DEV) for t in (q, k, v, sinks, d_out))
+            off = torch.tensor([24], dtype=torch.int32, device=DEV)
+            o0, lse0 = A.attention_forward(qd, kd, vd, sd, SCALE, w, 24)
+            o1, lse1 = A.attention_forward(qd, kd, vd, sd, SCALE, w, 3, q_offset_dev=off)
+            assert torch.equal(o0, o1) and torch.equal(lse0, lse1)
+            g0 = A.attention_backward(qd, kd, vd, sd, o0, lse0, dod, SCALE, w, 24)
+            g1 = A.attention_backward(qd, kd, vd, sd, o0, lse0, dod, SCALE, w, 3, q_offset_dev=off)
+            for x, y in zip(g0, g1):
+                assert torch.equal(x, y)
+            # autograd surface: a device tensor stays on the device, an int is passed by value
+            outs = []
+            for start in (torch.tensor(24, device=DEV), 24):
+                qq, kk, vv = (t.clone().requires_grad_(True) for t in (qd, kd, vd))
+                ss = sd.clone().requires_grad_(True)
+                o = A.attention(qq, kk, vv, ss, SCALE, w, start)
+                o.backward(dod)
+                outs.append((o, qq.grad, kk.grad, vv.grad, ss.grad))
+            for x, y in zip(*outs):
+                assert torch.equal(x, y)
+            assert torch.equal(outs[0][0], o0)
+
+
 def test_padded_small_batch(A):
     for w, lens in ((None, [77, 200]), (128, [300, 130]), (5, [1, 64])):
         s = max(lens)
