@@ -109,6 +109,21 @@ def test_small_shapes_vs_eager_oracle(A, b, h, g, s, w):
     compare_all(run_hip(A, *inp, w), oracle_eager(*inp, w))
 
 
+@pytest.mark.parametrize("b,h,g,s,w", [
+    (1, 32, 2, 700, 128),    # 16 query heads per KV head: the most the single-pass backward takes
+    (1, 24, 2, 450, 100),    # 12 per KV head, ragged last tile
+    (1, 17, 1, 200, 128),    # 17 per KV head: falls back to the dQ + dK/dV kernels
+    (2, 34, 2, 96, 128),     # the same with two batch rows and two KV heads
+    (2, 16, 8, 1000, 128),   # two batch rows, chunks of two tiles: every key tile sits on a seam
+    (1, 16, 2, 65, 128),     # a single chunk whose second tile holds one row
+    (1, 4, 2, 129, 1),       # window 1
+])
+def test_window_backward_group_sizes_and_seams(A, b, h, g, s, w):
+    print(f"case B={b} H={h} G={g} S={s} W={w}", flush=True)
+    inp = E.make_inputs(300 + s, b, h, g, s, 64, torch.bfloat16)
+    compare_all(run_hip(A, *inp, w), oracle_eager(*inp, w))
+
+
 @pytest.mark.parametrize("w", [None, 48])
 @pytest.mark.parametrize("gain,sink_shift", [(5.0, 0.0), (3.0, -300.0), (1.0, 200.0), (3.0, 90.0)])
 def test_wide_logit_range(A, w, gain, sink_shift):
