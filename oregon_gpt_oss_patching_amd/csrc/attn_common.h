@@ -162,7 +162,9 @@ __device__ __forceinline__ void tile_async(char *lds_tile, const bf16 *base, int
 }
 
 // The same copy with the lane-dependent part of the address precomputed: lane offsets (in
-// elements) of the wavefront's two 16-byte chunks relative to the tile's first row.  Only valid
+// bytes, so that the address is exactly (scalar pointer) + (zero-extended 32-bit register), the
+// form the instruction takes without any address arithmetic) of the wavefront's two 16-byte
+// chunks relative to the tile's first row.  Only valid
 // for tiles that lie completely inside the tensor (no row clamping); `tile` points at the
 // tile's first row and is wave-uniform, so the loads use scalar base + 32-bit lane offset.
 struct AsyncLaneOffsets { uint32_t off[2]; };
@@ -173,7 +175,7 @@ __device__ __forceinline__ AsyncLaneOffsets make_async_offsets(int64_t stride_s,
     for (int k = 0; k < 2; ++k) {
         const int r = 16 * w + 8 * k + (lane >> 3);
         const int c = (lane & 7) ^ swz(r);
-        o.off[k] = (uint32_t)(r * (int)stride_s + c * 8);
+        o.off[k] = (uint32_t)(r * (int)stride_s + c * 8) * 2u;
     }
     return o;
 }
@@ -181,7 +183,8 @@ __device__ __forceinline__ AsyncLaneOffsets make_async_offsets(int64_t stride_s,
 __device__ __forceinline__ void tile_async_inner(char *lds_tile, const bf16 *tile, const AsyncLaneOffsets &o, int w) {
 #pragma unroll
     for (int k = 0; k < 2; ++k)
-        __builtin_amdgcn_global_load_lds((glb_void_t *)(tile + o.off[k]), (lds_void_t *)(lds_tile + (16 * w + 8 * k) * kRowBytes), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((glb_void_t *)(reinterpret_cast<const char *>(tile) + o.off[k]),
+                                         (lds_void_t *)(lds_tile + (16 * w + 8 * k) * kRowBytes), 16, 0, 0);
 }
 
 // Waits until at most `n` of this wavefront's vector-memory operations are outstanding.
