@@ -1,8 +1,10 @@
 """gptoss_attn_bwd_static -- the backward that allocates nothing and brings its own scratch --
 against gptoss_attn_bwd on the same inputs, through the C ABI: two calls in a row on one GPU,
 the second on a smaller problem, so that what the first call left in the shared array is there
-when the second one runs.  Bit-for-bit where gptoss_attn_bwd does not cut key blocks into slices
-(window layers, long rows); at the bf16 tolerance of the parity tests where it does."""
+when the second one runs.  Bit-for-bit where gptoss_attn_bwd takes the same sums (dQ, dSinks; dK / dV
+of long full-causal rows); at the bf16 tolerance of the parity tests where it adds fp32 partial sums
+that the no-alloc variant has no room for (key blocks of short rows cut into slices, seam tiles
+between the chunks of a sliding-window layer)."""
 import ctypes
 
 import pytest
