@@ -335,10 +335,11 @@ __global__ __launch_bounds__(WinCfg::NWAVES * 64, 1) void attn_bwd_window_kernel
     int dead[1] = {0};
     const uint32_t ds_out0 = ds_store_addr(ds_base + pair * kStageTileBytes, 32 * sub + l32, half);
 
-    // ---- copies: wavefront 0 the Q tile, wavefront 1 the dO tile of each walk position (eight
-    // 16-byte-per-lane instructions), wavefront 2 the K and V rows of the next key tile ----
-    const int64_t lstride = (w == 0) ? a.qs.s : a.dos.s;
-    const int64_t ld_hstride = (w == 0) ? a.qs.h : a.dos.h;
+    // ---- copies: wavefront kWaveQ the Q tile, wavefront kWaveDO the dO tile of each walk position (eight
+    // 16-byte-per-lane instructions), wavefront kWaveTransit the K and V rows of the next key tile ----
+    constexpr int kWaveQ = 2, kWaveDO = 3, kWaveTransit = 0;   // the copying owners share their SIMDs with the (lighter) helpers
+    const int64_t lstride = (w == kWaveQ) ? a.qs.s : a.dos.s;
+    const int64_t ld_hstride = (w == kWaveQ) ? a.qs.h : a.dos.h;
     uint32_t ld_off[2];
     {
         const int lr = lane >> 3;
@@ -346,13 +347,13 @@ __global__ __launch_bounds__(WinCfg::NWAVES * 64, 1) void attn_bwd_window_kernel
         ld_off[1] = (uint32_t)(lr * (int)lstride + (((lane & 7) ^ swz(lr + 8)) * 8));
     }
     int iss_h = 0, iss_i0 = t0 * kTile;
-    const bf16 *ld_tile = (w == 0)
+    const bf16 *ld_tile = (w == kWaveQ)
         ? a.q + (int64_t)b * a.qs.b + (int64_t)(g * a.r) * a.qs.h + (int64_t)iss_i0 * a.qs.s
         : a.d_o + (int64_t)b * a.dos.b + (int64_t)(g * a.r) * a.dos.h + (int64_t)iss_i0 * a.dos.s;
     auto issue = [&](int it) {
         const int stage = it % NS;
-        if (w < 2) {
-            char *dst = smem + (stage * 2 + w) * kStageTileBytes;
+        if (w == kWaveQ || w == kWaveDO) {
+            char *dst = smem + (stage * 2 + (w - kWaveQ)) * kStageTileBytes;
             if (iss_i0 + kTile <= a.Sq) {
 #pragma unroll
                 for (int k = 0; k < 8; ++k)
@@ -404,11 +405,11 @@ __global__ __launch_bounds__(WinCfg::NWAVES * 64, 1) void attn_bwd_window_kernel
     auto iterate = [&](int it) {
         const int STAGE = stage;
         stage = stage == NS - 1 ? 0 : stage + 1;
-        if (w < 2) { if (it + 1 >= n_it) wait_vmcnt<0>(); else wait_vmcnt<8>(); }
-        else if (w == 2 && cur.h == 0) wait_vmcnt<0>();        // the transit copy of the key tile that starts now
+        if (w == kWaveQ || w == kWaveDO) { if (it + 1 >= n_it) wait_vmcnt<0>(); else wait_vmcnt<8>(); }
+        else if (w == kWaveTransit && cur.h == 0) wait_vmcnt<0>();        // the transit copy of the key tile that starts now
         __syncthreads();
         if (it + 2 < n_it) issue(it + 2);
-        if (w == 2 && cur.h == 1 && cur.t + 1 < t1) issue_transit(cur.t + 1);
+        if (w == kWaveTransit && cur.h == 1 && cur.t + 1 < t1) issue_transit(cur.t + 1);
 
         if (cur.h == 0 && cur.t > t0 && pair == cur.t % 3) {
             // this pair's key tile (cur.t - 3) is complete; take over key tile cur.t from the transit buffer
