@@ -124,6 +124,9 @@ __global__ __launch_bounds__(WinCfg::NWAVES * 64, 1) void attn_bwd_window_kernel
     }
 
     if (!owner) {
+        // the two helpers are the only wavefronts of their kind; whenever one of them can issue it goes
+        // before the owner it shares its SIMD with (measured: -4 % at S = 16384)
+        __builtin_amdgcn_s_setprio(1);
         // =================================== helper wavefronts ===================================
         const int hh = w - C::NOWN;
         const int srow = 32 * hh + (lane >> 1), hr = lane & 1;     // statistics: two lanes per row, 32 columns each
