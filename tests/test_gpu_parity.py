@@ -124,6 +124,29 @@ def test_window_backward_group_sizes_and_seams(A, b, h, g, s, w):
     compare_all(run_hip(A, *inp, w), oracle_eager(*inp, w))
 
 
+@pytest.mark.parametrize("scale", [0.1, 0.15, 1.0 / 3.0])
+@pytest.mark.parametrize("w", [None, 128])
+def test_softmax_scales_other_than_one_eighth(A, w, scale):
+    """Every other test runs at the GPT-OSS scale 1/8, a power of two; these scales are not.
+    dQ and dK grow with the scale (the softmax sharpens and the scale multiplies them), and with them
+    the absolute effect of rounding P and dS to bf16: rel-L2 stays at 2.5e-3 ... 3.3e-3 for scales from
+    0.1 to 1/3 while the absolute bound, written for the GPT-OSS scale, is passed at 1/5.  So the
+    largest scale is held to the relative bounds only."""
+    q, k, v, sinks, d_out = E.make_inputs(88, 1, 16, 2, 330, 64, torch.bfloat16)
+    qd, kd, vd, sd, dod = (t.to(DEV) for t in (q, k, v, sinks, d_out))
+    o, lse = A.attention_forward(qd, kd, vd, sd, scale, w)
+    dq, dk, dv, ds = A.attention_backward(qd, kd, vd, sd, o, lse, dod, scale, w)
+    f = [t.float() for t in (q, k, v, sinks, d_out)]
+    ro, rdq, rdk, rdv, rds = E.eager_attention_grads(*f, scale, w)
+    rlse = E.logsumexp_rows(f[0], f[1], f[3], scale, w)
+    if scale <= 0.15:
+        compare_all((o, lse, dq, dk, dv, ds), (ro, rlse, rdq, rdk, rdv, rds))
+    else:
+        assert float((lse.cpu() - rlse.float()).abs().max()) <= LSE_TOL
+        for name, g, r in zip(("o", "dq", "dk", "dv", "dsinks"), (o, dq, dk, dv, ds), (ro, rdq, rdk, rdv, rds)):
+            check(name, g, r, atol=None)
+
+
 @pytest.mark.parametrize("w", [None, 48])
 @pytest.mark.parametrize("gain,sink_shift", [(5.0, 0.0), (3.0, -300.0), (1.0, 200.0), (3.0, 90.0)])
 def test_wide_logit_range(A, w, gain, sink_shift):
