@@ -319,3 +319,36 @@ def test_hip_graph_capture_and_replay_match_eager_launches():
             torch.cuda.synchronize()
             for got, want in zip(outs, ref):
                 assert torch.equal(got, want)
+
+
+def test_hip_graph_replays_follow_a_query_offset_in_device_memory():
+    """A start position that lives in device memory is read by the kernels at run time, so one
+    captured graph serves different offsets: between replays only the int32 on the device changes
+    (the reference's kernels read their start_q tensor the same way, attention_kernel.py:44-47).
+    Every replay must equal the eager call with that offset passed by value."""
+    import oregon_gpt_oss_patching_amd as A
+    q, k, v, sinks, d_out = (t.to("cuda") for t in E.make_inputs(322, 1, 8, 2, 48, 64, torch.bfloat16, skv=160))
+    off = torch.zeros(1, dtype=torch.int32, device="cuda")
+    for window in (None, 32):
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):                      # warm-up on the capture stream
+            o, lse = A.attention_forward(q, k, v, sinks, 0.125, window, q_offset_dev=off)
+            A.attention_backward(q, k, v, sinks, o, lse, d_out, 0.125, window, q_offset_dev=off)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            o, lse = A.attention_forward(q, k, v, sinks, 0.125, window, q_offset_dev=off)
+            outs = (o, lse) + tuple(A.attention_backward(q, k, v, sinks, o, lse, d_out, 0.125, window, q_offset_dev=off))
+        for start in (112, 0, 57):
+            off.fill_(start)
+            for t in outs:
+                t.fill_(float("nan"))
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            o_ref, lse_ref = A.attention_forward(q, k, v, sinks, 0.125, window, start)
+            ref = (o_ref, lse_ref) + tuple(A.attention_backward(q, k, v, sinks, o_ref, lse_ref, d_out, 0.125, window, start))
+            for got, want in zip(outs, ref):
+                assert torch.equal(got, want), start
