@@ -174,12 +174,14 @@ int gptoss_attn_bwd_dq(const gptoss_attn_params *params, void *stream);
 /*
  * Whole backward on one stream, i.e. `_attention.backward`
  * (attention_kernel.py:276-344).  bf16 tensors take one of two routes:
- *   - sliding-window layers with window <= 128, Sq == Skv, q_offset == 0, no doc_start and
- *     2..64 query heads per KV head: ONE kernel that reads q, k, v, o, d_o once and produces dq,
- *     dk, dv and the dsinks terms from five matrix products per (query tile, key tile) pair
- *     (`_attn_bwd`'s own five dots, attention_kernel.py:199-217), the row statistics formed on
- *     the way; `delta` only holds a few dsinks partial sums.  Same values as steps 1-3 up to the
- *     order of the fp32 sums (differences in the last bf16 bit);
+ *   - sliding-window layers with window <= 128, Sq == Skv, q_offset == 0 (and no q_offset_dev), no
+ *     doc_start and 2..16 query heads per KV head: ONE kernel that reads q, k, v, o, d_o once and
+ *     produces dq, dk, dv and the dsinks terms from five matrix products per (query tile, key tile)
+ *     pair (`_attn_bwd`'s own five dots, attention_kernel.py:199-217), the row statistics formed
+ *     on the way, followed by a small kernel that adds the two fp32 shares of the key tiles on the
+ *     seams between workgroups and reduces dsinks; `delta` holds those shares and the dsinks
+ *     partial sums.  Same values as steps 1-3 up to the order of the fp32 sums (differences in
+ *     the last bf16 bit);
  *   - everything else: the dQ kernel computes delta and lse*log2(e) for its own rows (no
  *     separate pass over O and dO), stores them in `delta`, and the dSinks and dK/dV kernels
  *     follow: the same bits as steps 1-3 called one after the other.
@@ -199,7 +201,10 @@ int gptoss_attn_bwd(const gptoss_attn_params *params, void *stream);
  * refused with GPTOSS_ATTN_ERR_WORKSPACE before anything is launched.  Key blocks are never cut
  * into slices here (that needs a large scratch), so short full-causal bf16 problems run slower than
  * through gptoss_attn_bwd and their dK/dV may differ from it in the last bit (another summation
- * order); everything else is bit-identical (sliding-window layers take the same single-pass kernel).  Every call on one GPU uses that GPU's single array:
+ * order); sliding-window layers take the same single-pass kernel, but each workgroup walks two
+ * query tiles past its chunk instead of exchanging fp32 shares of the seam tiles (no room for
+ * them), so dK/dV of those tiles may differ in the last bit as well; dQ and dSinks are
+ * bit-identical.  Every call on one GPU uses that GPU's single array:
  * calls that overlap on one GPU (two streams, two threads) race; calls on one stream do not, and
  * nothing needs clearing between calls (every value read was written earlier in the same call).
  * The array stays resident on every GPU the library has run on until the process ends.
