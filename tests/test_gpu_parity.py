@@ -124,6 +124,23 @@ def test_window_backward_group_sizes_and_seams(A, b, h, g, s, w):
     compare_all(run_hip(A, *inp, w), oracle_eager(*inp, w))
 
 
+@pytest.mark.parametrize("lens", [[1300, 1], [64, 1300], [129, 640], [1299, 1300]])
+def test_window_backward_padded_rows_across_chunks(A, lens):
+    """Right-padded batch rows in a sliding-window layer: whole chunks of the single-pass backward
+    (and the seams between them) lie in the padding of the shorter row; padded positions must come
+    out exactly zero and the valid ones match the oracle."""
+    b, h, g, s, w = 2, 16, 4, 1300, 128
+    q, k, v, sinks, d_out = E.make_inputs(500 + lens[0], b, h, g, s, 64, torch.bfloat16)
+    d_out = mask_dout(d_out, lens)
+    got = run_hip(A, q, k, v, sinks, d_out, w, 0, lens)
+    compare_all(got, oracle_eager(q, k, v, sinks, d_out, w, 0, lens))
+    o, lse, dq, dk, dv, ds = got
+    for i, n in enumerate(lens):
+        if n < s:
+            for t in (dq, dk, dv):
+                assert float(t[i, :, n:].abs().max()) == 0.0
+
+
 @pytest.mark.parametrize("scale", [0.1, 0.15, 1.0 / 3.0])
 @pytest.mark.parametrize("w", [None, 128])
 def test_softmax_scales_other_than_one_eighth(A, w, scale):
