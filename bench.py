@@ -314,7 +314,7 @@ def cpu_model():
 
 def cpu_baseline(s, d, scale):
     """Eager fp32 restatement (forward + autograd backward) on the host cores, on a bounded
-    sample: two query heads sharing one KV head of the full-causal layer.  Threads: what torch
+    sample: two calls of four query heads sharing one KV head of the full-causal layer.  Threads: what torch
     was given (OMP_NUM_THREADS / the CPU share of the box), never more than the host reports."""
     import torch
     from oracle import eager_ref as E

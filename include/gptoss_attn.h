@@ -9,9 +9,10 @@
  * Conventions
  *   - plain pointers and sizes only; no torch, no HIP types (the stream is passed
  *     as a void* holding a hipStream_t; NULL is the default stream);
- *   - every buffer is owned by the caller; the library allocates nothing and
- *     keeps no mutable global state, so calls on different streams are
- *     independent;
+ *   - every buffer is owned by the caller; the library allocates nothing.  Its only
+ *     process-wide state is per-device values that are looked up once and never change
+ *     (compute-unit count, a kernel attribute, the address of the built-in scratch of
+ *     gptoss_attn_bwd_static), so calls on different streams are independent;
  *   - launches are asynchronous on `stream`; no entry point synchronises;
  *   - outputs need no pre-zeroing (the reference needs dk/dv/dsinks zeroed,
  *     attention_kernel.py:296-298; this library writes every element once);
@@ -135,7 +136,11 @@ const char *gptoss_attn_status_string(int status);
  * GPU (bf16, full-causal, short sequences), the fp32 partial dK / dV sums of the slices each key
  * block is cut into.  The reference allocates its counterpart itself
  * (`delta = torch.empty_like(M)`, attention_kernel.py:303) and accumulates dK / dV with atomics
- * (:204,212); here the caller owns the scratch and the sums are taken in a fixed order.  Host-only.
+ * (:204,212); here the caller owns the scratch and the sums are taken in a fixed order.  For the
+ * sliding-window layers that gptoss_attn_bwd runs as one kernel the same bytes hold that kernel's
+ * dSinks partial sums and the fp32 dK / dV shares of the key tiles on the seams between workgroups;
+ * how many seams there are depends on the compute-unit count of the device the launch runs on, and
+ * the size returned covers the largest number any device can ask for.  Host-only: no HIP call.
  */
 size_t gptoss_attn_workspace_bytes(const gptoss_attn_params *params);
 

@@ -59,6 +59,7 @@ struct WinCfg {
     static constexpr int kLdsBytes = kSinkOff + NHELP * kMaxGroup * 64 * 4;
     static_assert(kDsOff % 128 == 0 && kTransitOff % 128 == 0, "swizzled tiles start on 128-byte boundaries");
     static_assert(kLdsBytes <= 160 * 1024, "one workgroup per CU");
+    static_assert(kMaxGroup * NHELP * 64 * 4 == kLdsBytes - kSinkOff, "the dSinks slots in LDS bound the query heads per KV head");
 };
 
 // (query tile, head within the group) of a position of the walk

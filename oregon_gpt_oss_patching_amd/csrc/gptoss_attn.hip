@@ -1,6 +1,7 @@
 // C ABI of the gfx950 GPT-OSS attention library (declared in include/gptoss_attn.h):
 // host-side argument validation, launch geometry, and the kernel launches.
-// No torch headers, no allocation, no global mutable state.
+// No torch headers, no allocation; the only process-wide state is three per-device caches that are
+// written once (compute-unit count, the window kernel's LDS attribute, the address of the built-in scratch).
 #include <hip/hip_runtime.h>
 
 #include <atomic>
@@ -117,7 +118,8 @@ int launch(Kernel kernel, int64_t workgroups, int threads, hipStream_t st, const
 
 // ---- single-pass backward of sliding-window layers (attn_bwd_window.h) ------------------------
 // Taken for bf16 self-attention (Sq == Skv, no offset, no packed rows) with a window of at most
-// 128 and 2..64 query heads per KV head; everything else keeps the dK/dV + dQ kernel pair.
+// 128 and 2..16 query heads per KV head (WinCfg::kMaxGroup: the kernel's LDS holds dSinks slots for
+// that many); everything else keeps the dK/dV + dQ kernel pair.
 bool window_single_pass(const gptoss_attn_params *p) {
     const int r = p->G > 0 ? p->H / p->G : 0;
     const int window = effective_window(p);
@@ -168,15 +170,17 @@ int window_lds_attribute() {
 // to 16 bytes) the fp32 dK / dV shares of the two key tiles on each seam between chunks.
 struct WindowScratch { int chunk_tiles, n_chunks; size_t sink_bytes, seam_bytes; };
 
-WindowScratch window_scratch(const gptoss_attn_params *p, int cus) {
+WindowScratch window_scratch_for(const gptoss_attn_params *p, int chunk_tiles) {
     WindowScratch w;
-    w.chunk_tiles = window_chunk_tiles(p, cus);
+    w.chunk_tiles = chunk_tiles;
     const int n_tiles = (p->Sq + kTile - 1) / kTile;
     w.n_chunks = (n_tiles + w.chunk_tiles - 1) / w.chunk_tiles;
     w.sink_bytes = (((size_t)p->B * w.n_chunks * p->H * WinCfg::NHELP * sizeof(float)) + 15) & ~(size_t)15;
     w.seam_bytes = (size_t)p->B * p->G * (w.n_chunks - 1) * 2 * 2 * (2 * kTile * kD) * sizeof(float);
     return w;
 }
+
+WindowScratch window_scratch(const gptoss_attn_params *p, int cus) { return window_scratch_for(p, window_chunk_tiles(p, cus)); }
 
 // seam_sums: neighbouring chunks exchange fp32 shares through the scratch (needs window_scratch bytes);
 // otherwise each chunk walks two query tiles past its end and nothing but the dSinks sums is kept.
@@ -276,8 +280,10 @@ size_t gptoss_attn_workspace_bytes(const gptoss_attn_params *p) {
         const int parts = dkdv_parts_for(p);
         if (parts > 1) n += (size_t)parts * 2 * sizeof(float) * (size_t)p->B * (size_t)p->G * (size_t)p->Skv * kD;
         if (window_single_pass(p)) {
-            // gptoss_attn_bwd takes this route and lays its own scratch over the same bytes
-            const WindowScratch ws = window_scratch(p, compute_units());
+            // gptoss_attn_bwd takes this route and lays its own scratch over the same bytes.  The layout
+            // follows the compute-unit count of the device that is current at launch time; the size
+            // returned is that of the shortest chunks (the most seams), which covers every device.
+            const WindowScratch ws = window_scratch_for(p, 2);
             if (ws.sink_bytes + ws.seam_bytes > n) n = ws.sink_bytes + ws.seam_bytes;
         }
     }

@@ -50,6 +50,40 @@ def test_struct_mirror_matches_header_field_order():
     assert ctypes.sizeof(_lib.Params) == 360
 
 
+def _integration_stub_classes():
+    """The ctypes classes of the binding stub that INTEGRATION.md shows a maintainer, executed as
+    they stand in that file."""
+    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    block = next(b for b in re.findall(r"```python\n(.*?)```", text, re.S) if "class Params(ctypes.Structure)" in b)
+    start = block.index("class Strides(ctypes.Structure)")
+    end = block.index("lib = ctypes.CDLL")
+    ns = {"ctypes": ctypes}
+    exec(block[start:end], ns)
+    return ns["Strides"], ns["Params"]
+
+
+def test_integration_doc_stub_matches_the_library():
+    """The documented reference-side binding must be accepted by the shipped library: same size,
+    same field names, offsets and sizes as the package's own mirror, and a block filled through it
+    passes validation."""
+    strides_cls, params_cls = _integration_stub_classes()
+    assert ctypes.sizeof(strides_cls) == ctypes.sizeof(_lib.Strides)
+    assert ctypes.sizeof(params_cls) == ctypes.sizeof(_lib.Params) == 360
+    assert [f[0] for f in params_cls._fields_] == [f[0] for f in _lib.Params._fields_]
+    for name, _ in _lib.Params._fields_:
+        mine, doc = getattr(_lib.Params, name), getattr(params_cls, name)
+        assert (mine.offset, mine.size) == (doc.offset, doc.size), name
+    good = _valid_params()
+    p = params_cls.from_buffer_copy(bytes(good))
+    p.struct_size = ctypes.sizeof(params_cls)
+    lib = ctypes.CDLL(_lib.LIBRARY)
+    lib.gptoss_attn_validate.restype = ctypes.c_int
+    assert lib.gptoss_attn_validate(ctypes.byref(p), 1) == 0
+    assert lib.gptoss_attn_version() == 4
+    for name in ("gptoss_attn_fwd", "gptoss_attn_bwd", "gptoss_attn_bwd_static"):   # what the stub binds
+        assert getattr(lib, name) is not None
+
+
 def _valid_params():
     """A parameter block that passes validation (fake, aligned, never dereferenced)."""
     p = _lib.new_params()
@@ -182,8 +216,8 @@ def test_workspace_bytes():
     assert lib.gptoss_attn_workspace_bytes(ctypes.byref(p)) == stats + 4 * 2 * 4 * 1 * 8 * 4096 * 64
     # a sliding-window layer the single-pass backward takes: its dSinks partial sums [B][chunks][H][2]
     # and 128 KB of fp32 dK/dV shares per (batch, KV head, seam between chunks), if that is more than
-    # the row statistics.  64 query tiles x 8 KV heads over 256 compute units (the count assumed
-    # without a device, and MI355X's) = 2 tiles per chunk, 32 chunks.
+    # the row statistics.  The size is that of the shortest chunks any device can ask for (2 query
+    # tiles), so it does not depend on the device: 64 query tiles = 32 chunks.
     p.window = 128
     chunks = 32
     assert lib.gptoss_attn_workspace_bytes(ctypes.byref(p)) == 1 * chunks * 64 * 2 * 4 + 1 * 8 * (chunks - 1) * 128 * 1024
