@@ -18,17 +18,22 @@ SCALE = 0.125
 DEV = "cuda"
 
 
-def _backward_both(b, h, g, s, window, seed):
+def _backward_both(b, h, g, s, window, seed, dtype=torch.bfloat16, lens=None):
     from oregon_gpt_oss_patching_amd import _lib
     from oregon_gpt_oss_patching_amd import attention_kernel as ak
     lib = _lib.load()
-    q, k, v, sinks, d_out = (t.to(DEV) for t in E.make_inputs(seed, b, h, g, s, 64, torch.bfloat16))
-    o, lse = ak.attention_forward(q, k, v, sinks, SCALE, window)
+    q, k, v, sinks, d_out = E.make_inputs(seed, b, h, g, s, 64, dtype)
+    if lens is not None:
+        qvalid = (torch.arange(s).view(1, s) < torch.tensor(lens).view(b, 1)).view(b, s, 1, 1)
+        d_out = d_out * qvalid
+    q, k, v, sinks, d_out = (t.to(DEV) for t in (q, k, v, sinks, d_out))
+    sl = None if lens is None else torch.tensor(lens, dtype=torch.int32, device=DEV)
+    o, lse = ak.attention_forward(q, k, v, sinks, SCALE, window, 0, lens)
     s32 = sinks.float().contiguous()
     stream = torch.cuda.current_stream().cuda_stream
     results = []
     for name in ("gptoss_attn_bwd", "gptoss_attn_bwd_static"):
-        p = ak._base_params(q, k, v, s32, None, SCALE, window, 0)
+        p = ak._base_params(q, k, v, s32, sl, SCALE, window, 0)
         p.o, p.lse, p.d_o = o.data_ptr(), lse.data_ptr(), d_out.data_ptr()
         ak._set(p.o_stride, ak._strides_bhs(o, "bshd"))
         ak._set(p.do_stride, ak._strides_bhs(d_out, "bshd"))
@@ -79,6 +84,32 @@ def test_static_scratch_backward_matches_workspace_backward(window):
     print(f"no-alloc backward, window={window}: second call B=1 H=8 G=2 S=333 (smaller)", flush=True)
     ref, got, cut = _backward_both(1, 8, 2, 333, window, 12)
     _compare(ref, got, cut)
+
+
+@pytest.mark.parametrize("b,h,g,s,window,dtype,lens", [
+    (2, 8, 2, 300, None, torch.float32, None),           # float32 tensors: preprocess + dK/dV + dQ on the built-in scratch
+    (2, 8, 2, 300, 64, torch.float32, [300, 1]),
+    (2, 16, 4, 1300, 128, torch.bfloat16, [1300, 1]),    # padded rows in the window kernel's walk past its chunk:
+    (2, 16, 4, 1300, 128, torch.bfloat16, [64, 1300]),   # whole chunks and their neighbour tiles lie in the padding
+    (2, 16, 4, 1300, 128, torch.bfloat16, [1299, 129]),
+    (1, 17, 1, 200, 128, torch.bfloat16, None),          # 17 query heads per KV head: dQ + dK/dV kernels, static scratch
+    (1, 4, 4, 200, 128, torch.bfloat16, None),           # one query head per KV head: the same fallback
+    (2, 17, 1, 200, None, torch.bfloat16, [200, 77]),
+])
+def test_static_scratch_backward_other_routes(b, h, g, s, window, dtype, lens):
+    """The routes the two-call test above does not take, each against gptoss_attn_bwd: float32 tensors,
+    right-padded rows in the single-pass window kernel's no-seam walk (every workgroup walks two query
+    tiles past its chunk and drops the dK/dV of the two tiles before it), and group sizes the
+    single-pass kernel does not take.  Padded positions must be exactly zero."""
+    print(f"no-alloc backward: B={b} H={h} G={g} S={s} W={window} {dtype} lens={lens}", flush=True)
+    ref, got, cut = _backward_both(b, h, g, s, window, 13, dtype, lens)
+    single_pass = dtype == torch.bfloat16 and window is not None and window <= 128 and 2 <= h // g <= 16
+    _compare(ref, got, cut or single_pass)
+    if lens is not None:
+        for i, n in enumerate(lens):
+            if n < s:
+                for t in got[:3]:
+                    assert float(t[i, :, n:].abs().max()) == 0.0
 
 
 def test_static_scratch_refuses_what_does_not_fit():
