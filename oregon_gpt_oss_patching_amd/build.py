@@ -21,6 +21,9 @@ HIPCC_FLAGS = [
     "-shared",
     # packed fp32 VALU ops are kept off for every kernel in this library
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # MFMA results stay in ordinary vector registers unless a kernel pins an accumulator to the AGPR half
+    # itself (the 64-key dK/dV kernel does, through inline assembly)
+    "-mllvm", "-amdgpu-mfma-vgpr-form",
 ]
 
 

@@ -106,6 +106,34 @@ __device__ __forceinline__ void ds_store_zero(uint32_t base, int qb) {
     ds_store(base, qb, 1, z);
 }
 
+// ---- MFMAs whose accumulator lives in the AGPR half of the register file -----------------------------
+// A kernel that runs one wavefront per SIMD has 512 registers per lane, 256 of them AGPRs, which only
+// MFMAs (and copies) can touch.  The compiler keeps all MFMA results of a kernel in one kind of register;
+// the library is built so that this is the VGPR kind (the vector instructions of the softmax read S and
+// dP), and the long-lived dK / dV accumulators of attn_bwd_dkdv64_kernel are kept in AGPRs through these
+// inline-assembly MFMAs.  What the compiler cannot see inside the assembly, and the callers therefore
+// guarantee themselves:
+//   * an operand written by a vector instruction is at least two instructions old when the MFMA reads it
+//     (SAFE pays for that itself with two wait states);
+//   * no other instruction reads an accumulator sooner than an MFMA takes to finish, not even a
+//     register-to-register copy, which the compiler may place wherever two pieces of straight-line code
+//     meet (it does move the accumulators between the pipelined loop and the code around it): the last
+//     of these MFMAs in such a piece is followed by eight or more ordinary MFMAs or by
+//     agpr_accumulators_settled(), and the first one in a piece is the SAFE form (a copy is a vector
+//     instruction too).  tests/test_isa_dkdv64.py checks the compiled kernel for this.
+template <bool SAFE>
+__device__ __forceinline__ void mfma_bf16_agpr(f32x16 &acc, const bf16x8 a, const bf16x8 b) {
+    if constexpr (SAFE) asm("s_nop 1\n\tv_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+    else asm("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc) : "v"(a), "v"(b));
+}
+// Longer than the 16 passes of the slowest MFMA.  The accumulators are operands, so they are still where
+// the MFMAs left them when the delay starts and anything the compiler does with them comes after it.
+__device__ __forceinline__ void agpr_accumulators_settled(f32x16 (&dk)[2][2], f32x16 (&dv)[2][2]) {
+    asm volatile("s_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15\n\ts_nop 15"
+                 : "+a"(dv[0][0]), "+a"(dv[0][1]), "+a"(dv[1][0]), "+a"(dv[1][1]), "+a"(dk[0][0]), "+a"(dk[0][1]), "+a"(dk[1][0]),
+                   "+a"(dk[1][1]));
+}
+
 // ---------------------------------------------------------------------------------
 // dK, dV.  Workgroup = NW wavefronts x 64 keys of KV head g, batch b.  The K and V
 // rows of a wavefront stay in registers as MFMA B operands (two 32-key blocks, so
@@ -127,7 +155,7 @@ __device__ __forceinline__ void ds_store_zero(uint32_t base, int qb) {
 // 128-byte row of 64 query-row columns per key, 16-byte chunks XOR-swizzled like every staged
 // tile.  A 32-row block that is skipped stores zeros.  The wavefronts that form dQ read it back
 // with the transposing fragment reads.
-template <bool MASKED, bool DOCS, int NB, bool STORE_DS = false>
+template <bool MASKED, bool DOCS, int NB, bool STORE_DS = false, bool AGPR_ACC = false, bool STAT_BLOCKED = false>
 __device__ __forceinline__ void dkdv_tile(uint32_t qsm, uint32_t gsm, uint32_t stat_lane, const TileLaneOffsets &lo,
                                           const bf16x8 (&kf)[NB][4], const bf16x8 (&vf)[NB][4],
                                           f32x16 (&dk)[NB][2], f32x16 (&dv)[NB][2], float c, int half,
@@ -167,7 +195,8 @@ __device__ __forceinline__ void dkdv_tile(uint32_t qsm, uint32_t gsm, uint32_t s
             // the dP accumulators start at -delta of their rows, so the MFMAs deliver dP - delta
 #pragma unroll
             for (int a4 = 0; a4 < 4; ++a4) {
-                const f32x4 nd = lds_load128f(stat_lane, (kTile + 32 * qb + 8 * a4) * 4);
+                // STAT_BLOCKED: per 32-row block, 32 values of lse2 followed by its 32 values of -delta
+                const f32x4 nd = lds_load128f(stat_lane, (STAT_BLOCKED ? 64 * qb + 32 + 8 * a4 : kTile + 32 * qb + 8 * a4) * 4);
 #pragma unroll
                 for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
@@ -185,7 +214,7 @@ __device__ __forceinline__ void dkdv_tile(uint32_t qsm, uint32_t gsm, uint32_t s
         }
 #pragma unroll
         for (int a4 = 0; a4 < 4; ++a4) {
-            const f32x4 lv = lds_load128f(stat_lane, (32 * qb + 8 * a4) * 4);
+            const f32x4 lv = lds_load128f(stat_lane, (STAT_BLOCKED ? 64 * qb + 8 * a4 : 32 * qb + 8 * a4) * 4);
             u32x4 dsr = {0u, 0u, 0u, 0u};
             if (MASKED && DOCS) dsr = lds_load128(ds_lane, (32 * qb + 8 * a4) * 4);
 #pragma unroll
@@ -223,8 +252,13 @@ __device__ __forceinline__ void dkdv_tile(uint32_t qsm, uint32_t gsm, uint32_t s
                 if constexpr (STORE_DS) ds_store(ds_out, qb, u, dsf);
 #pragma unroll
                 for (int dblk = 0; dblk < 2; ++dblk) {
-                    dv[nb][dblk] = mfma_bf16(agt[dblk], pf, dv[nb][dblk]);
-                    dk[nb][dblk] = mfma_bf16(aqt[dblk], dsf, dk[nb][dblk]);
+                    if constexpr (AGPR_ACC) {      // the accumulators are pinned to AGPRs (attn_bwd_dkdv64_kernel)
+                        mfma_bf16_agpr<true>(dv[nb][dblk], agt[dblk], pf);
+                        mfma_bf16_agpr<true>(dk[nb][dblk], aqt[dblk], dsf);
+                    } else {
+                        dv[nb][dblk] = mfma_bf16(agt[dblk], pf, dv[nb][dblk]);
+                        dk[nb][dblk] = mfma_bf16(aqt[dblk], dsf, dk[nb][dblk]);
+                    }
                 }
             }
         }

@@ -5,9 +5,11 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <cstdlib>
 
 #include "../../include/gptoss_attn.h"
 #include "attn_bwd.h"
+#include "attn_bwd_dkdv64.h"
 #include "attn_bwd_window.h"
 #include "attn_common.h"
 #include "attn_f32.h"
@@ -326,8 +328,12 @@ static int launch_dkdv(const gptoss_attn_params *p, void *stream, bool whole_blo
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (p->dtype == GPTOSS_ATTN_FP32)
         return launch(attn_f32_dkdv_kernel, f32_grid((int64_t)a.B * a.G * ((a.Skv + 31) / 32)), 256, st, a);
-    a.dkdv_parts = whole_blocks ? 1 : dkdv_parts_for(p);
+    a.dkdv_parts = (whole_blocks || getenv("GPTOSS_DKDV_WHOLE")) ? 1 : dkdv_parts_for(p);
     a.dkdv_partial = reinterpret_cast<float *>(reinterpret_cast<char *>(p->delta) + stats_bytes(p));
+    if (getenv("GPTOSS_DKDV_NB2") && !a.doc_start && a.dkdv_parts == 1 && a.Sq % 64 == 0) {   // EXPERIMENT
+        const int64_t grid2 = (int64_t)a.G * a.B * ((a.Skv + 255) / 256);
+        return launch(attn_bwd_dkdv64_kernel, grid2, 256, st, a);
+    }
     const int64_t grid = (int64_t)a.G * a.B * a.dkdv_parts * ((a.Skv + kDkdvKeys - 1) / kDkdvKeys);
     const int s = a.doc_start ? launch(attn_bwd_dkdv_kernel<kDkdvWaves, kDkdvNB, true>, grid, 64 * kDkdvWaves, st, a)
                               : launch(attn_bwd_dkdv_kernel<kDkdvWaves, kDkdvNB, false>, grid, 64 * kDkdvWaves, st, a);
