@@ -11,9 +11,11 @@ import subprocess
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 SOURCE = os.path.join(_HERE, "csrc", "gptoss_attn.hip")
-LIBRARY = os.path.join(_HERE, "libgptoss_attn.so")
+LIBRARY = os.environ.get("GPTOSS_LIB_OUT") or os.path.join(_HERE, "libgptoss_attn.so")
 
 HIPCC_FLAGS = [
+    *(["-DGPTOSS_DKDV_TIMING"] if __import__("os").environ.get("GPTOSS_TIMING") else []),
+    *(__import__("os").environ.get("GPTOSS_DEFS", "").split()),
     "--offload-arch=gfx950",
     "-O3",
     "-std=c++17",

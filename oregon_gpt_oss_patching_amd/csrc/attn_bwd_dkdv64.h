@@ -268,18 +268,26 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv64_kernel(const KArgs a) 
         constexpr int RKIND = decltype(rkind_)::value, RQB = decltype(rqb_)::value;
         constexpr bool SYNC = decltype(sync_)::value;
         constexpr int TV = (TC + 3) & 3;     // the substep whose last two steps are finished here
+#ifndef GPTOSS_ABL_NOSYNC
         if constexpr (SYNC) { arrive(); GPTOSS_FENCE(); }
+#endif
 #pragma unroll
         for (int m = 0; m < 16; ++m) {
             if (m < 8) m2(TP, m); else m1(TN, m - 8);
+#ifndef GPTOSS_ABL_NOV
             if (m < 2) vstep(std::false_type{}, TV, 16 + m);
             vstep(masked_, TC, m);
+#endif
+#ifndef GPTOSS_ABL_NOLDS
             if (RKIND == 1) rd(st, stl, RQB, (m + 8) & 15);
             if (RKIND == 2 && (m & 1) == 0) rd(st, stl, RQB, 16 + (m >> 1));
+#endif
+#ifndef GPTOSS_ABL_NODMA
             if constexpr (SYNC) {
                 if (m >= 2 && m < 2 + C::kCopiesPerTile) issue_one(m - 2);
                 if (m == 2 + C::kCopiesPerTile) advance();
             }
+#endif
             GPTOSS_FENCE();
         }
     };
@@ -302,12 +310,21 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv64_kernel(const KArgs a) 
         issue();
     }
     // one tile through the four slots (A..D of the header comment)
+#ifdef GPTOSS_DKDV_TIMING
+    uint64_t tsl[8] = {0, 0, 0, 0, 0, 0, 0, 0}, tprev = 0;
+#define GPTOSS_TS(kk) { const uint64_t tnow = __builtin_readcyclecounter(); if (tprev) tsl[kk] += tnow - tprev; tprev = tnow; }
+#else
+#define GPTOSS_TS(kk)
+#endif
     auto body = [&](auto masked_, uint32_t st, uint32_t stl, uint32_t nst, uint32_t nstl) __attribute__((always_inline)) {
+        GPTOSS_TS(4)
         GPTOSS_FENCE();
         // slot A: M2(3 of the tile before), M1(1) | V(0) | block 1: statistics, natural fragments
         slot(masked_, I1{}, I3{}, I0{}, I1{}, I1{}, F{}, st, stl);
+        GPTOSS_TS(0)
         // slot B: M2(0), M1(2) | V(1) | block 1: transposed fragments
         slot(masked_, I2{}, I0{}, I1{}, I2{}, I1{}, F{}, st, stl);
+        GPTOSS_TS(1)
         // slot C: the next tile has landed (and this one's stage is free for the request after next);
         //         M2(1), M1(3) | V(2) | next tile, block 0: statistics, natural fragments
         // slot D: M2(2), M1(0 of the next tile) | V(3) | next tile, block 0: transposed fragments
@@ -315,21 +332,21 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv64_kernel(const KArgs a) 
         // staged data of a tile this wavefront skips, or a repeated copy after the last tile.  Its results
         // are never used; the body stays free of variants and branches.)
         slot(masked_, I3{}, I1{}, I2{}, I1{}, I0{}, T{}, nst, nstl);
+        GPTOSS_TS(2)
         slot(masked_, I0{}, I2{}, I3{}, I2{}, I0{}, F{}, nst, nstl);
+        GPTOSS_TS(3)
+#ifdef GPTOSS_DKDV_TIMING
+        tsl[5] += 1;
+#endif
     };
 
+    // A full-causal walk without padded rows (what the host sends here) meets, per wavefront: interior tiles,
+    // then the masked tile(s) on the diagonal, then tiles whose rows all precede the wavefront's keys.  The
+    // kernel is laid out as exactly that, one piece after the other with no loop around them.
     int k = 0;
     int cls = n_it > 0 ? classify(cur_i0) : kSkip;
-    while (k < n_it) {
-        if (cls == kSkip) {
-            ++k;
-            cur_stage = next_stage(cur_stage);
-            if (++cur_h == a.r) { cur_h = 0; cur_i0 -= kTile; cls = k < n_it ? classify(cur_i0) : kSkip; }
-            arrive();
-            issue();
-            continue;
-        }
-        // ---- a run of tiles through the pipeline ----
+    if (cls != kSkip) {
+        // ---- the tiles that do something, through the pipeline ----
         {   // fill: block 0 of the first tile, M1(0).  The first slot of the loop also issues M2 of "the tile
             // before": for the first tile of a run that is a product of zeros (exact: the accumulators keep
             // their bits), which keeps the loop body free of variants.
@@ -373,6 +390,10 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv64_kernel(const KArgs a) 
             cls = ncls;
             live = has_next && ncls != kSkip;
         };
+        // (The explicit waits in front of the loops: whatever loads the compiler itself has in flight here,
+        // reloads of spilled registers included, are then known to have arrived, and it puts no vmcnt wait of
+        // its own into the loops, where it would drain the copies in flight on every pass.)
+        wait_vmcnt<0>();
         while (live && cls == kInterior) step_tile(F{});
         if (live && cls == kMasked) {
             const int pos0 = q_offset + cur_i0;          // masked tiles that follow one another belong to one query tile
@@ -385,6 +406,7 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv64_kernel(const KArgs a) 
                 mwd[nb] = (unsigned)max(0, min(weff, mdb[nb] + max(row_lim, -8) - 4 * half));
             }
             const int i0_masked = cur_i0;
+            wait_vmcnt<0>();
             while (live && cls == kMasked && cur_i0 == i0_masked) step_tile(T{});
         }
         // drain: the tail of V(3) and M2(3)
@@ -396,8 +418,20 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv64_kernel(const KArgs a) 
         for (int j = 0; j < 8; ++j) m2(3, j);
         agpr_accumulators_settled(dk, dv);
     }
+    // ---- the rest of the walk: nothing to compute, but every wavefront keeps the workgroup's rhythm of
+    // barriers and requests ----
+    for (; k < n_it; ++k) {
+        arrive();
+        issue();
+    }
 #undef GPTOSS_FENCE
 
+#ifdef GPTOSS_DKDV_TIMING
+    if (lane == 0 && blockIdx.x < 64) {
+        float *dbg = a.delta + 2 * (int64_t)a.B * a.H * a.Sq + (blockIdx.x * 4 + w) * 8;
+        for (int i = 0; i < 8; ++i) dbg[i] = (float)tsl[i];
+    }
+#endif
     wait_vmcnt<0>();          // the repeated copies of the last requests
     agpr_accumulators_settled(dk, dv);
     if (a.dkdv_parts > 1) {

@@ -330,7 +330,7 @@ static int launch_dkdv(const gptoss_attn_params *p, void *stream, bool whole_blo
         return launch(attn_f32_dkdv_kernel, f32_grid((int64_t)a.B * a.G * ((a.Skv + 31) / 32)), 256, st, a);
     a.dkdv_parts = (whole_blocks || getenv("GPTOSS_DKDV_WHOLE")) ? 1 : dkdv_parts_for(p);
     a.dkdv_partial = reinterpret_cast<float *>(reinterpret_cast<char *>(p->delta) + stats_bytes(p));
-    if (getenv("GPTOSS_DKDV_NB2") && !a.doc_start && a.dkdv_parts == 1 && a.Sq % 64 == 0) {   // EXPERIMENT
+    if (getenv("GPTOSS_DKDV_NB2") && !a.doc_start && !a.seqlens && a.window == 0 && a.dkdv_parts == 1 && a.Sq % 64 == 0) {   // EXPERIMENT
         const int64_t grid2 = (int64_t)a.G * a.B * ((a.Skv + 255) / 256);
         return launch(attn_bwd_dkdv64_kernel, grid2, 256, st, a);
     }
