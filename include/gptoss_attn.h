@@ -28,7 +28,8 @@
  *                through the same (b, h, s) stride triple, so any layout works
  *   lse          (B, H, Sq) fp32 contiguous
  *   delta        fp32 scratch of gptoss_attn_workspace_bytes() bytes, 16-byte aligned: -rowsum(dO*O), then
- *                lse*log2(e), then (short sequences) partial dK/dV sums
+ *                lse*log2(e), then both once more as 16 bytes per row of bf16 terms for the dK/dV
+ *                kernels, then (short sequences) partial dK/dV sums
  *   sinks, dsinks (H,) fp32;  sinks == NULL means a sink logit of 0, as in the
  *                reference (attention_kernel.py:39-42)
  *   seqlens      (B,) int32 or NULL: right-padding lengths.  Keys at or beyond
@@ -75,12 +76,12 @@ enum gptoss_attn_status {
     GPTOSS_ATTN_ERR_ALIGNMENT = -7,     /* a tensor base or stride breaks 16-byte row alignment */
     GPTOSS_ATTN_ERR_STRIDE = -8,        /* a sequence stride smaller than D or larger than 2^24 elements */
     GPTOSS_ATTN_ERR_ABI = -9,           /* struct_size does not match this library */
-    GPTOSS_ATTN_ERR_WORKSPACE = -10     /* gptoss_attn_bwd_static: 2*B*H*Sq floats do not fit the built-in scratch */
+    GPTOSS_ATTN_ERR_WORKSPACE = -10     /* gptoss_attn_bwd_static: 24*B*H*Sq bytes do not fit the built-in scratch */
 };
 
-/* Size of the device array gptoss_attn_bwd_static keeps its row statistics in: 2*B*H*Sq floats must
+/* Size of the device array gptoss_attn_bwd_static keeps its row statistics in: 24 bytes per row must
  * fit, i.e. B*H*Sq <= 2 097 152 rows (the 64-head layer at S = 16384 is 1 048 576 rows per batch row). */
-#define GPTOSS_ATTN_STATIC_SCRATCH_BYTES (16u << 20)
+#define GPTOSS_ATTN_STATIC_SCRATCH_BYTES (48u << 20)
 
 /* (batch, head, sequence) strides in elements. */
 typedef struct gptoss_attn_strides {
@@ -132,7 +133,9 @@ const char *gptoss_attn_status_string(int status);
 /*
  * Bytes of the `delta` scratch buffer the backward entry points need for these shapes; 0 for a
  * NULL or shapeless params.  Reads dtype, B, H, G, Sq, Skv and window.  The buffer holds
- * 2 * B * H * Sq floats of row statistics and, when the problem has too few key blocks to fill the
+ * 24 bytes of row statistics per (batch, head, query row): 2 * B * H * Sq floats, and the same numbers
+ * (lse / scale and -delta) each split into three bf16 terms, which the dK/dV kernels feed to the matrix
+ * pipe as one more step of their S and dP products.  When the problem has too few key blocks to fill the
  * GPU (bf16, full-causal, short sequences), the fp32 partial dK / dV sums of the slices each key
  * block is cut into.  The reference allocates its counterpart itself
  * (`delta = torch.empty_like(M)`, attention_kernel.py:303) and accumulates dK / dV with atomics
@@ -155,7 +158,9 @@ int gptoss_attn_fwd(const gptoss_attn_params *params, void *stream);
 /*
  * Backward step 1: the row statistics.  The first B*H*Sq floats of `delta` receive
  * -rowsum(dO * O) (the NEGATED row dot: it seeds the dP accumulators of the kernels that
- * follow), the next B*H*Sq floats lse * log2(e).  Replaces `_attn_bwd_precompute_D`
+ * follow), the next B*H*Sq floats lse * log2(e); behind them (from the next 16-byte boundary) 16
+ * bytes per row hold lse / scale and the negated row dot as three bf16 terms each, the form the dK/dV
+ * kernels read.  Replaces `_attn_bwd_precompute_D`
  * (attention_kernel.py:102-120, 304-313) including the dO transpose copy at
  * :290.  When dsinks != NULL it also produces
  * dsinks[h] = -sum_{b,i} exp(sinks[h] - lse) * delta   (attention_kernel.py:173-176)
@@ -186,7 +191,8 @@ int gptoss_attn_bwd_dq(const gptoss_attn_params *params, void *stream);
  *     on the way, followed by a small kernel that adds the two fp32 shares of the key tiles on the
  *     seams between workgroups and reduces dsinks; `delta` holds those shares and the dsinks
  *     partial sums.  Same values as steps 1-3 up to the order of the fp32 sums (differences in
- *     the last bf16 bit);
+ *     the last bf16 bit, and of the rare P or dS value that rounds to the other bf16 neighbour
+ *     because the dK/dV kernels of steps 1-3 subtract lse inside the matrix product);
  *   - everything else: the dQ kernel computes delta and lse*log2(e) for its own rows (no
  *     separate pass over O and dO), stores them in `delta`, and the dSinks and dK/dV kernels
  *     follow: the same bits as steps 1-3 called one after the other.

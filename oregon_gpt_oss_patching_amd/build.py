@@ -14,7 +14,6 @@ SOURCE = os.path.join(_HERE, "csrc", "gptoss_attn.hip")
 LIBRARY = os.environ.get("GPTOSS_LIB_OUT") or os.path.join(_HERE, "libgptoss_attn.so")
 
 HIPCC_FLAGS = [
-    *(["-DGPTOSS_DKDV_TIMING"] if __import__("os").environ.get("GPTOSS_TIMING") else []),
     *(__import__("os").environ.get("GPTOSS_DEFS", "").split()),
     "--offload-arch=gfx950",
     "-O3",

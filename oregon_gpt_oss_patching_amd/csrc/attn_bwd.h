@@ -19,7 +19,8 @@ namespace gptoss {
 // load it straight into the dP accumulators).  HBM-bound stream: eight lanes
 // read one 128-byte row of each tensor, reduce with three xor-shuffles.  The same
 // pass stores lse*log2(e) in the second half of the scratch buffer, which is what
-// the dK/dV and dQ kernels feed to exp2.
+// the dQ and dSinks kernels feed to exp2, and both statistics once more in the split form the
+// dK/dV kernels take (split_row_stats).
 __global__ __launch_bounds__(256) void attn_bwd_delta_kernel(const KArgs a) {
     constexpr int kRowsPerThread = 4;                      // independent 128-bit loads in flight per tensor
     const int64_t total = (int64_t)a.B * a.H * a.Sq;       // rows, indexed (b*H + h)*Sq + s
@@ -52,6 +53,7 @@ __global__ __launch_bounds__(256) void attn_bwd_delta_kernel(const KArgs a) {
         if (c == 0 && rid < total) {
             a.delta[rid] = -acc;                          // stored negated: it seeds the dP accumulators
             a.delta[total + rid] = a.lse[rid] * kLog2e;   // second half of the scratch: lse in log2 units
+            a.split[rid] = split_row_stats(a.lse[rid], a.scale, -acc);
         }
     }
 }
@@ -155,7 +157,9 @@ __device__ __forceinline__ void agpr_accumulators_settled(f32x16 (&dk)[2][2], f3
 // 128-byte row of 64 query-row columns per key, 16-byte chunks XOR-swizzled like every staged
 // tile.  A 32-row block that is skipped stores zeros.  The wavefronts that form dQ read it back
 // with the transposing fragment reads.
-template <bool MASKED, bool DOCS, int NB, bool STORE_DS = false, bool AGPR_ACC = false, bool STAT_BLOCKED = false>
+// SPLIT: the row statistics are staged in the split form (split_row_stats) and enter through one more
+// step of the S and dP contractions; stat_lane then addresses the 16 bytes of row l32 of block 0.
+template <bool MASKED, bool DOCS, int NB, bool STORE_DS = false, bool SPLIT = false>
 __device__ __forceinline__ void dkdv_tile(uint32_t qsm, uint32_t gsm, uint32_t stat_lane, const TileLaneOffsets &lo,
                                           const bf16x8 (&kf)[NB][4], const bf16x8 (&vf)[NB][4],
                                           f32x16 (&dk)[NB][2], f32x16 (&dv)[NB][2], float c, int half,
@@ -178,7 +182,9 @@ __device__ __forceinline__ void dkdv_tile(uint32_t qsm, uint32_t gsm, uint32_t s
             width[nb] = (unsigned)max(0, min((int)weff, dbh[nb] + max(row_lim, -8) - 4 * half));
         }
     }
-    // qsm / gsm: LDS byte addresses of the staged Q and dO tiles; stat_lane: address of this
+    bf16x8 b_stat_s, b_stat_dp;
+    if constexpr (SPLIT) stat_step_operands(half, b_stat_s, b_stat_dp);
+    // qsm / gsm: LDS byte addresses of the staged Q and dO tiles; stat_lane (not SPLIT): address of this
     // lane's first lse2 value (rows 4*half..), -delta sits kTile floats further on.
     // DOCS (packed rows): ds_lane addresses the staged document starts of the same rows, jkey
     // is the lane's key index; a key before its query's document start is invisible.
@@ -192,16 +198,27 @@ __device__ __forceinline__ void dkdv_tile(uint32_t qsm, uint32_t gsm, uint32_t s
             continue;
         }
         f32x16 s[NB], dp[NB];
+        if constexpr (SPLIT) {
+            // the statistics step: S starts at -lse / scale, dP at -delta of the rows
+            const bf16x8 a_stat = as_bf16x8(lds_load128(stat_lane, 32 * qb * 16));
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+                for (int i = 0; i < 16; ++i) { s[nb][i] = 0.0f; dp[nb][i] = 0.0f; }
+                s[nb] = mfma_bf16(a_stat, b_stat_s, s[nb]);
+                dp[nb] = mfma_bf16(a_stat, b_stat_dp, dp[nb]);
+            }
+        } else {
             // the dP accumulators start at -delta of their rows, so the MFMAs deliver dP - delta
 #pragma unroll
             for (int a4 = 0; a4 < 4; ++a4) {
-                // STAT_BLOCKED: per 32-row block, 32 values of lse2 followed by its 32 values of -delta
-                const f32x4 nd = lds_load128f(stat_lane, (STAT_BLOCKED ? 64 * qb + 32 + 8 * a4 : kTile + 32 * qb + 8 * a4) * 4);
+                const f32x4 nd = lds_load128f(stat_lane, (kTile + 32 * qb + 8 * a4) * 4);
 #pragma unroll
                 for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
                     for (int e = 0; e < 4; ++e) { s[nb][4 * a4 + e] = 0.0f; dp[nb][4 * a4 + e] = nd[e]; }
             }
+        }
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) {
             const bf16x8 aq = ofrag_nat(qsm, lo, qb, ks);
@@ -214,7 +231,8 @@ __device__ __forceinline__ void dkdv_tile(uint32_t qsm, uint32_t gsm, uint32_t s
         }
 #pragma unroll
         for (int a4 = 0; a4 < 4; ++a4) {
-            const f32x4 lv = lds_load128f(stat_lane, (STAT_BLOCKED ? 64 * qb + 8 * a4 : 32 * qb + 8 * a4) * 4);
+            f32x4 lv = {0.0f, 0.0f, 0.0f, 0.0f};
+            if constexpr (!SPLIT) lv = lds_load128f(stat_lane, (32 * qb + 8 * a4) * 4);
             u32x4 dsr = {0u, 0u, 0u, 0u};
             if (MASKED && DOCS) dsr = lds_load128(ds_lane, (32 * qb + 8 * a4) * 4);
 #pragma unroll
@@ -222,7 +240,7 @@ __device__ __forceinline__ void dkdv_tile(uint32_t qsm, uint32_t gsm, uint32_t s
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int i = 4 * a4 + e;
-                    float pe = fast_exp2(fmaf(s[nb][i], c, -lv[e]));
+                    float pe = fast_exp2(SPLIT ? s[nb][i] * c : fmaf(s[nb][i], c, -lv[e]));
                     if (MASKED) {
                         bool vis;
                         if constexpr (STORE_DS) {
@@ -252,13 +270,8 @@ __device__ __forceinline__ void dkdv_tile(uint32_t qsm, uint32_t gsm, uint32_t s
                 if constexpr (STORE_DS) ds_store(ds_out, qb, u, dsf);
 #pragma unroll
                 for (int dblk = 0; dblk < 2; ++dblk) {
-                    if constexpr (AGPR_ACC) {      // the accumulators are pinned to AGPRs (attn_bwd_dkdv64_kernel)
-                        mfma_bf16_agpr<true>(dv[nb][dblk], agt[dblk], pf);
-                        mfma_bf16_agpr<true>(dk[nb][dblk], aqt[dblk], dsf);
-                    } else {
-                        dv[nb][dblk] = mfma_bf16(agt[dblk], pf, dv[nb][dblk]);
-                        dk[nb][dblk] = mfma_bf16(aqt[dblk], dsf, dk[nb][dblk]);
-                    }
+                    dv[nb][dblk] = mfma_bf16(agt[dblk], pf, dv[nb][dblk]);
+                    dk[nb][dblk] = mfma_bf16(aqt[dblk], dsf, dk[nb][dblk]);
                 }
             }
         }
@@ -273,7 +286,7 @@ __global__ __launch_bounds__(NW * 64, (NB == 1 ? 2 : 1)) void attn_bwd_dkdv_kern
     constexpr int WK = 32 * NB;        // keys per wavefront
     constexpr int BN = WK * NW;        // keys per workgroup
     __shared__ __attribute__((aligned(16))) char smem[NS][2][kStageTileBytes];
-    __shared__ __attribute__((aligned(16))) float sstat[NS][2][kTile];
+    __shared__ __attribute__((aligned(16))) u32x4 sstat[NS][kTile];               // split row statistics of the staged rows
     __shared__ __attribute__((aligned(16))) int32_t sdoc[DOCS ? NS : 1][kTile];   // document starts of the staged rows
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
@@ -337,9 +350,8 @@ __global__ __launch_bounds__(NW * 64, (NB == 1 ? 2 : 1)) void attn_bwd_dkdv_kern
     int dead[NB];
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) dead[nb] = 0;
-    const float *lse2 = a.delta + (int64_t)a.B * a.H * a.Sq;   // written by the delta kernel
     const TileLaneOffsets lo = make_tile_offsets(lane);
-    const uint32_t smem_base = lds_addr(&smem[0][0][0]), stat_base = lds_addr(&sstat[0][0][0]);
+    const uint32_t smem_base = lds_addr(&smem[0][0][0]), stat_base = lds_addr(&sstat[0][0]);
     const uint32_t doc_base = lds_addr(&sdoc[0][0]);
     constexpr bool has_docs = DOCS;
     int jkey[NB];
@@ -356,25 +368,25 @@ __global__ __launch_bounds__(NW * 64, (NB == 1 ? 2 : 1)) void attn_bwd_dkdv_kern
     const bf16 *qtile = a.q + (int64_t)b * a.qs.b + (int64_t)(g * a.r) * a.qs.h + (int64_t)iss_i0 * a.qs.s;
     const bf16 *gtile = a.d_o + (int64_t)b * a.dos.b + (int64_t)(g * a.r) * a.dos.h + (int64_t)iss_i0 * a.dos.s;
     int64_t stat_off = ((int64_t)b * a.H + (int64_t)g * a.r) * a.Sq + iss_i0;    // (b, head, row) of the tile's first row
-    // wavefront w copies 32 floats of lse2 (w < 2) or delta (w >= 2) per tile; 16 document starts
-    const float *stat_lane = ((w >> 1) ? a.delta : lse2) + 32 * (w & 1) + (lane & 31);
+    // wavefront w copies the statistics of 16 rows (16 bytes each) per tile, and 16 document starts
+    const u32x4 *stat_lane = a.split + 16 * w + (lane & 15);
     const int32_t *doc_lane = DOCS ? a.doc_start + (int64_t)b * a.Sq + 16 * w + (lane & 15) : nullptr;
     auto issue = [&](int it) {
         const int stage = it % NS;
         if (iss_i0 + kTile <= a.Sq) {
             tile_async_inner(smem[stage][0], qtile, qlane, w);
             tile_async_inner(smem[stage][1], gtile, glane, w);
-            if (lane < 32)
-                __builtin_amdgcn_global_load_lds((glb_void_t *)(stat_lane + stat_off), (lds_void_t *)(&sstat[stage][w >> 1][32 * (w & 1)]), 4, 0, 0);
+            if (lane < 16)
+                __builtin_amdgcn_global_load_lds((glb_void_t *)(stat_lane + stat_off), (lds_void_t *)(&sstat[stage][16 * w]), 16, 0, 0);
             if (DOCS && lane < 16)
                 __builtin_amdgcn_global_load_lds((glb_void_t *)(doc_lane + iss_i0), (lds_void_t *)(&sdoc[DOCS ? stage : 0][16 * w]), 4, 0, 0);
         } else {
             // the tile sticks out of the tensor: rows past the end re-read the last valid one
             tile_async(smem[stage][0], qtile - (int64_t)iss_i0 * a.qs.s, a.qs.s, iss_i0, a.Sq, lane, w);
             tile_async(smem[stage][1], gtile - (int64_t)iss_i0 * a.dos.s, a.dos.s, iss_i0, a.Sq, lane, w);
-            if (lane < 32) {
-                const int over = max(0, iss_i0 + 32 * (w & 1) + lane - (a.Sq - 1));
-                __builtin_amdgcn_global_load_lds((glb_void_t *)(stat_lane + stat_off - over), (lds_void_t *)(&sstat[stage][w >> 1][32 * (w & 1)]), 4, 0, 0);
+            if (lane < 16) {
+                const int over = max(0, iss_i0 + 16 * w + lane - (a.Sq - 1));
+                __builtin_amdgcn_global_load_lds((glb_void_t *)(stat_lane + stat_off - over), (lds_void_t *)(&sstat[stage][16 * w]), 16, 0, 0);
             }
             if (DOCS && lane < 16) {
                 const int over = max(0, iss_i0 + 16 * w + lane - (a.Sq - 1));
@@ -407,7 +419,7 @@ __global__ __launch_bounds__(NW * 64, (NB == 1 ? 2 : 1)) void attn_bwd_dkdv_kern
         if (it + 2 < n_it) issue(it + 2);
 
         const uint32_t qsm = smem_base + STAGE * (2 * kStageTileBytes), gsm = qsm + kStageTileBytes;
-        const uint32_t stat_lane = stat_base + STAGE * (2 * kTile * 4) + half * 16;
+        const uint32_t stat_lane = stat_base + STAGE * (kTile * 16) + l32 * 16;
         const uint32_t ds_lane = doc_base + STAGE * (kTile * 4) + half * 16;
         const int i0 = cur_i0;
         if (++cur_h == a.r) { cur_h = 0; cur_i0 -= kTile; }
@@ -427,7 +439,7 @@ __global__ __launch_bounds__(NW * 64, (NB == 1 ? 2 : 1)) void attn_bwd_dkdv_kern
         }
         if (skip) return;
         if (interior) {
-            dkdv_tile<false, false, NB>(qsm, gsm, stat_lane, lo, kf, vf, dk, dv, c, half, dead, 0u, 0, 0, 0u, jkey);
+            dkdv_tile<false, false, NB, false, true>(qsm, gsm, stat_lane, lo, kf, vf, dk, dv, c, half, dead, 0u, 0, 0, 0u, jkey);
         } else {
             int dbase[NB];
 #pragma unroll
@@ -436,7 +448,7 @@ __global__ __launch_bounds__(NW * 64, (NB == 1 ? 2 : 1)) void attn_bwd_dkdv_kern
                 dbase[nb] = (j < kv_len) ? pos0 - j : -0x40000000;
             }
             const int row_lim = (int)min((int64_t)kTile, min((int64_t)a.Sq, (int64_t)q_len - q_offset) - i0);
-            dkdv_tile<true, DOCS, NB>(qsm, gsm, stat_lane, lo, kf, vf, dk, dv, c, half, dbase, (unsigned)weff, row_lim,
+            dkdv_tile<true, DOCS, NB, false, true>(qsm, gsm, stat_lane, lo, kf, vf, dk, dv, c, half, dbase, (unsigned)weff, row_lim,
                                       wj0 - pos0, ds_lane, jkey);
         }
     };
@@ -680,6 +692,7 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_bwd_dq_kernel(co
                 if (half == 0 && active) {
                     a.delta[off] = dlt[qb];
                     a.delta[(int64_t)a.B * a.H * a.Sq + off] = lse2[qb];
+                    a.split[off] = split_row_stats(a.lse[off], a.scale, dlt[qb]);
                 }
             }
         } else if (row_ok) {

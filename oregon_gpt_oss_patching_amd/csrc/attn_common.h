@@ -43,7 +43,8 @@ struct KArgs {
     const bf16 *d_o;
     bf16 *dq, *dk, *dv;
     float *dsinks;
-    float *delta;
+    float *delta;        // row statistics in fp32: -delta[B][H][Sq], then lse * log2(e) [B][H][Sq]
+    u32x4 *split;        // the same statistics as bf16 triples, 16 bytes per row (see split_row_stats)
     Strides qs, ks, vs, os, dos, dqs, dks, dvs;
     int B, H, G, Sq, Skv;
     int r;               // H / G query heads per KV head
@@ -79,6 +80,41 @@ __device__ __forceinline__ bf16x8 as_bf16x8(const u32x4 v) {
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// ---- row statistics as an MFMA operand -----------------------------------------------------------
+// The dK/dV kernels need, for every element of a 32 x 32 block of S and dP, a number that belongs to the
+// element's ROW (lse and delta), while a lane of the MFMA result holds one COLUMN: read as they are, the
+// statistics cost eight broadcast LDS reads per block.  Instead they enter through the matrix pipe as one
+// more step of the contraction: the A operand of that step holds, per row, L = lse / scale and -delta, each
+// split into three bf16 terms whose sum is the fp32 value (3 x 8 mantissa bits; the products with +-1 are
+// exact and the accumulation is fp32), and the B operand holds -1 against the terms of L (for S) or +1
+// against the terms of -delta (for dP), so that the MFMAs deliver S - L and dP - delta and
+// P = exp2((S - L) * scale * log2(e)).
+//   row layout (8 bf16): L_hi, L_mid, L_lo, 0, nd_hi, nd_mid, nd_lo, 0
+__device__ __forceinline__ void split3_bf16(float x, uint32_t &w01, uint32_t &w2) {
+    union { bf16 h; uint16_t u; } hi, mid, lo;
+    hi.h = (bf16)x;
+    const float r1 = x - (float)hi.h;       // exact
+    mid.h = (bf16)r1;
+    const float r2 = r1 - (float)mid.h;     // exact
+    lo.h = (bf16)r2;
+    w01 = (uint32_t)hi.u | ((uint32_t)mid.u << 16);
+    w2 = (uint32_t)lo.u;
+}
+__device__ __forceinline__ u32x4 split_row_stats(float lse, float scale, float neg_delta) {
+    uint32_t w0, w1, w2, w3;
+    split3_bf16(lse / scale, w0, w1);
+    split3_bf16(neg_delta, w2, w3);
+    return u32x4{w0, w1, w2, w3};
+}
+// B operands of the statistics step; only the lanes of half 0 carry k = 0..7 of the 16-deep step, and the
+// A operand repeats the row's 16 bytes in both halves (finite times zero)
+__device__ __forceinline__ void stat_step_operands(int half, bf16x8 &b_s, bf16x8 &b_dp) {
+    const u32x4 s = {half ? 0u : 0xBF80BF80u, half ? 0u : 0x0000BF80u, 0u, 0u};
+    const u32x4 d = {0u, 0u, half ? 0u : 0x3F803F80u, half ? 0u : 0x00003F80u};
+    b_s = as_bf16x8(s);
+    b_dp = as_bf16x8(d);
+}
 // max(a, b) as median(a, b, +inf): one v_med3_f32, without the NaN-quieting pre-pass that
 // fmaxf costs in IEEE mode (the kernels never produce NaN: masked logits are -inf and the
 // running max is finite).
@@ -159,9 +195,20 @@ typedef __attribute__((address_space(1))) const void glb_void_t;
 __device__ __forceinline__ void lds_dma16(uint32_t lds_base, const void *gbase, uint32_t voff) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(voff), "s"(gbase) : "memory");
 }
+// the same with the LDS base given as (scalar register) + (compile-time constant): one scalar instruction
+// forms the sum in M0
+template <int IMM>
+__device__ __forceinline__ void lds_dma16_plus(uint32_t lds_base, const void *gbase, uint32_t voff) {
+    if constexpr (IMM == 0) lds_dma16(lds_base, gbase, voff);
+    else asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(voff), "s"(gbase), "n"(IMM) : "memory", "scc");
+}
 // the same with a full per-lane address
 __device__ __forceinline__ void lds_dma16_at(uint32_t lds_base, const void *gaddr) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(gaddr) : "memory");
+}
+// lane L's 4 bytes at gbase + voff land at lds_base + 4 * L
+__device__ __forceinline__ void lds_dma4(uint32_t lds_base, const void *gbase, uint32_t voff) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds_base), "v"(voff), "s"(gbase) : "memory");
 }
 // lane L's 4 bytes at gaddr land at lds_base + 4 * L
 __device__ __forceinline__ void lds_dma4_at(uint32_t lds_base, const void *gaddr) {

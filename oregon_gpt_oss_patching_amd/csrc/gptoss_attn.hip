@@ -5,7 +5,6 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
-#include <cstdlib>
 
 #include "../../include/gptoss_attn.h"
 #include "attn_bwd.h"
@@ -41,6 +40,13 @@ int effective_window(const gptoss_attn_params *p) {
     return (p->window > 0 && (int64_t)p->window >= (int64_t)p->Sq + p->q_offset) ? 0 : p->window;
 }
 
+// Scratch layout: the fp32 row statistics (-delta, then lse * log2 e: 8 bytes per row, rounded up to 16
+// bytes), the same statistics in split form (16 bytes per row), then the dK/dV partial sums.
+size_t fp32_stats_bytes(const gptoss_attn_params *p) {
+    const size_t n = (size_t)2 * sizeof(float) * (size_t)p->B * (size_t)p->H * (size_t)p->Sq;
+    return (n + 15) & ~(size_t)15;
+}
+
 KArgs make_args(const gptoss_attn_params *p) {
     KArgs a{};
     a.q = static_cast<const bf16 *>(p->q);
@@ -57,6 +63,7 @@ KArgs make_args(const gptoss_attn_params *p) {
     a.dv = static_cast<bf16 *>(p->dv);
     a.dsinks = p->dsinks;
     a.delta = p->delta;
+    a.split = reinterpret_cast<u32x4 *>(reinterpret_cast<char *>(p->delta) + fp32_stats_bytes(p));
     a.qs = cvt(p->q_stride); a.ks = cvt(p->k_stride); a.vs = cvt(p->v_stride); a.os = cvt(p->o_stride);
     a.dos = cvt(p->do_stride); a.dqs = cvt(p->dq_stride); a.dks = cvt(p->dk_stride); a.dvs = cvt(p->dv_stride);
     a.B = p->B; a.H = p->H; a.G = p->G; a.Sq = p->Sq; a.Skv = p->Skv;
@@ -101,6 +108,16 @@ int dkdv_parts_for(const gptoss_attn_params *p) {
     if (parts > tiles / 4) parts = tiles / 4;
     if (parts > 8) parts = 8;
     return parts < 1 ? 1 : parts;
+}
+
+// Long full-causal self-attention rows go to attn_bwd_dkdv64_kernel (64 keys per wavefront, one wavefront
+// per SIMD): bf16, no window, no padded or packed rows, no offset, Sq == Skv a multiple of 64, and enough
+// key blocks that the 32-key kernel would not cut them into slices (then the 256-key workgroups of the
+// 64-key kernel are at least 257, one per compute unit and more).  Same bits as the 32-key kernel.
+bool dkdv64_route(const gptoss_attn_params *p) {
+    const int64_t blocks = (int64_t)p->G * p->B * ((p->Skv + kDkdvKeys - 1) / kDkdvKeys);
+    return p->dtype == GPTOSS_ATTN_BF16 && effective_window(p) == 0 && !p->seqlens && !p->doc_start && p->q_offset == 0 &&
+           !p->q_offset_dev && p->Sq == p->Skv && p->Sq % kTile == 0 && blocks > 512;
 }
 
 // workgroups of four independent wavefronts for the float32 kernels
@@ -269,10 +286,9 @@ int gptoss_attn_validate(const gptoss_attn_params *p, int need_bwd) {
     return GPTOSS_ATTN_OK;
 }
 
-// Bytes of the row-statistics part of the scratch (rounded up to 16 bytes); dK/dV partials follow.
+// Bytes of the row-statistics part of the scratch; dK/dV partials follow.
 static size_t stats_bytes(const gptoss_attn_params *p) {
-    const size_t n = (size_t)2 * sizeof(float) * (size_t)p->B * (size_t)p->H * (size_t)p->Sq;
-    return (n + 15) & ~(size_t)15;
+    return fp32_stats_bytes(p) + (size_t)16 * (size_t)p->B * (size_t)p->H * (size_t)p->Sq;
 }
 
 size_t gptoss_attn_workspace_bytes(const gptoss_attn_params *p) {
@@ -328,12 +344,9 @@ static int launch_dkdv(const gptoss_attn_params *p, void *stream, bool whole_blo
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (p->dtype == GPTOSS_ATTN_FP32)
         return launch(attn_f32_dkdv_kernel, f32_grid((int64_t)a.B * a.G * ((a.Skv + 31) / 32)), 256, st, a);
-    a.dkdv_parts = (whole_blocks || getenv("GPTOSS_DKDV_WHOLE")) ? 1 : dkdv_parts_for(p);
+    if (dkdv64_route(p)) return launch(attn_bwd_dkdv64_kernel, (int64_t)a.G * a.B * ((a.Skv + Dkdv64::BN - 1) / Dkdv64::BN), 256, st, a);
+    a.dkdv_parts = whole_blocks ? 1 : dkdv_parts_for(p);
     a.dkdv_partial = reinterpret_cast<float *>(reinterpret_cast<char *>(p->delta) + stats_bytes(p));
-    if (getenv("GPTOSS_DKDV_NB2") && !a.doc_start && !a.seqlens && a.window == 0 && a.dkdv_parts == 1 && a.Sq % 64 == 0) {   // EXPERIMENT
-        const int64_t grid2 = (int64_t)a.G * a.B * ((a.Skv + 255) / 256);
-        return launch(attn_bwd_dkdv64_kernel, grid2, 256, st, a);
-    }
     const int64_t grid = (int64_t)a.G * a.B * a.dkdv_parts * ((a.Skv + kDkdvKeys - 1) / kDkdvKeys);
     const int s = a.doc_start ? launch(attn_bwd_dkdv_kernel<kDkdvWaves, kDkdvNB, true>, grid, 64 * kDkdvWaves, st, a)
                               : launch(attn_bwd_dkdv_kernel<kDkdvWaves, kDkdvNB, false>, grid, 64 * kDkdvWaves, st, a);

@@ -206,13 +206,15 @@ def test_validate_float32_params_and_their_alignment_rule():
 def test_workspace_bytes():
     lib = _lib.load()
     p = _valid_params()
-    assert lib.gptoss_attn_workspace_bytes(ctypes.byref(p)) == 2 * 4 * 1 * 8 * 128
+    # row statistics: -delta and lse * log2(e) in fp32 (8 bytes per row), then both again as the bf16 triples
+    # the dK/dV kernels feed to the matrix pipe (16 bytes per row)
+    assert lib.gptoss_attn_workspace_bytes(ctypes.byref(p)) == (8 + 16) * 1 * 8 * 128
     p.B, p.H, p.G, p.Sq, p.Skv = 4, 64, 8, 16384, 16384
-    assert lib.gptoss_attn_workspace_bytes(ctypes.byref(p)) == 2 * 4 * 4 * 64 * 16384
+    assert lib.gptoss_attn_workspace_bytes(ctypes.byref(p)) == (8 + 16) * 4 * 64 * 16384
     # short sequences: the dK/dV kernel cuts each key block's query tiles into slices (here 4) and
     # keeps their fp32 partial sums behind the row statistics; sliding-window layers are never cut
     p.B, p.Sq, p.Skv = 1, 4096, 4096
-    stats = 2 * 4 * 1 * 64 * 4096
+    stats = (8 + 16) * 1 * 64 * 4096
     assert lib.gptoss_attn_workspace_bytes(ctypes.byref(p)) == stats + 4 * 2 * 4 * 1 * 8 * 4096 * 64
     # a sliding-window layer the single-pass backward takes: its dSinks partial sums [B][chunks][H][2]
     # and 128 KB of fp32 dK/dV shares per (batch, KV head, seam between chunks), if that is more than

@@ -188,3 +188,51 @@ def test_sweep_misses_are_the_bf16_rounding_of_p(A, seed, b, h, g, s, w, atol):
         # arithmetic: one such flip moves an output by ulp(p) * |dO| or ulp(dS) * |q| * scale, a few 1e-3
         assert excess <= RECOMPUTE_EXCESS, (name, excess)
         assert off <= 0.01, (name, off)
+
+
+# ---- the 64-key dK/dV kernel (long full-causal rows) ------------------------------------------------
+# gptoss_attn_bwd sends bf16 full-causal self-attention without padded or packed rows, Sq a multiple of 64
+# and more than 512 key blocks of 128 to attn_bwd_dkdv64_kernel.  Many short batch rows reach that route
+# at sizes the CPU oracle still handles.
+
+DKDV64_CASES = [
+    # B, H, G, S
+    (17, 8, 4, 1024),      # two query heads per KV head, four 256-key workgroups per row
+    (16, 8, 4, 1088),      # S = 4 * 256 + 64: the last workgroup of a row has one live wavefront
+    (9, 8, 8, 1024),       # one query head per KV head
+    (12, 18, 6, 960),      # three per KV head, S = 3 * 256 + 192
+    (130, 4, 4, 64),       # one tile: every wavefront but the first idles
+]
+
+
+@pytest.mark.parametrize("b,h,g,s", DKDV64_CASES)
+def test_dkdv64_route_vs_eager_oracle(A, b, h, g, s):
+    assert g * b * ((s + 127) // 128) > 512 and s % 64 == 0      # the route's own condition
+    print(f"case B={b} H={h} G={g} S={s}", flush=True)
+    inp = E.make_inputs(1500 + s + b, b, h, g, s, 64, torch.bfloat16)
+    got = TP.run_hip(A, *inp, None)
+    o, lse, dq, dk, dv, ds = (t.detach().cpu() for t in got)
+    # the oracle one batch row at a time (dSinks adds up over the rows)
+    rds = torch.zeros(h, dtype=torch.float64)
+    for i in range(b):
+        one = [t[i:i + 1] for t in (inp[0], inp[1], inp[2])] + [inp[3], inp[4][i:i + 1]]
+        ro, rlse, rdq, rdk, rdv, rds_i = TP.oracle_eager(*one, None)
+        TP.compare_all((o[i:i + 1], lse[i:i + 1], dq[i:i + 1], dk[i:i + 1], dv[i:i + 1], rds_i), (ro, rlse, rdq, rdk, rdv, rds_i))
+        rds += rds_i.double()
+    TP.check("dsinks", ds, rds.float(), atol=None)
+
+
+@pytest.mark.parametrize("b,h,g,s", [(1, 64, 8, 16384), (3, 16, 8, 8192 + 64), (16, 8, 4, 1088)])
+def test_dkdv64_route_has_the_bits_of_the_32_key_kernel(A, b, h, g, s):
+    """The same problem with a seqlens array that pads nothing takes attn_bwd_dkdv_kernel (32 keys per
+    wavefront, the general kernel): both add the same products in the same order, so dK and dV agree bit
+    for bit, at GPT-OSS-20B's full 16384-token layer too."""
+    print(f"case B={b} H={h} G={g} S={s}", flush=True)
+    q, k, v, sinks, d_out = (t.to(DEV) for t in E.make_inputs(1700 + s, b, h, g, s, 64, torch.bfloat16))
+    o, lse = A.attention_forward(q, k, v, sinks, SCALE, None)
+    one = A.attention_backward(q, k, v, sinks, o, lse, d_out, SCALE, None)
+    two = A.attention_backward(q, k, v, sinks, o, lse, d_out, SCALE, None, 0, [s] * b)
+    torch.cuda.synchronize()
+    for name, x, y in zip(("dq", "dk", "dv", "dsinks"), one, two):
+        assert torch.isfinite(x.float()).all(), name
+        assert torch.equal(x, y), name
