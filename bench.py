@@ -239,7 +239,7 @@ def main():
     bytes_bwd = 2 * B * S * D * (4 * H + 4 * G) + 12 * B * H * S
     bytes_total = bytes_fwd + bytes_bwd
 
-    # dominant kernel: dkdv computes S, dP, dV, dK = 4 of the 7 algorithmic GEMMs
+    # dominant kernel: dK/dV (attn_bwd_dkdv64_kernel at this shape) computes S, dP, dV, dK = 4 of the 7 algorithmic GEMMs
     dkdv_ms = kern["full.bwd_dkdv"]
     dkdv_tflops = 4 * unit / (dkdv_ms * 1e-3) / 1e12
     win_bwd_ms = kern["win128.bwd"]
@@ -291,13 +291,13 @@ def main():
         "kernel_ms": kern,
         "other_configs": other,
         "device": device_info(),
-        "roofline": {"bound": "mfma", "kernel": "attn_bwd_dkdv_kernel (full causal)",
+        "roofline": {"bound": "mfma", "kernel": "attn_bwd_dkdv64_kernel (full causal)",
                      "achieved": round(dkdv_tflops, 2), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(dkdv_tflops / PEAK_BF16_TFLOPS, 4),
                      # HBM bytes per launch of this kernel at S=16384 from the committed rocprofv3 counter record
                      # (FETCH_SIZE and WRITE_SIZE scaled by a plain 1 GiB copy); null when that record was taken
                      # with other kernel sources
-                     "traffic": recorded_traffic("attn_bwd_dkdv_kernel", "full") if S == 16384 else None},
+                     "traffic": recorded_traffic("attn_bwd_dkdv64_kernel", "full") if S == 16384 else None},
     }
 
     if not args.no_cpu_baseline:
@@ -423,7 +423,7 @@ def summarize(dirs, layer, out_md):
     """Reads the *_results.db of each directory, prints / writes a text summary and records the
     HBM bytes per launch (FETCH_SIZE, WRITE_SIZE scaled by what the 1 GiB calibration copy shows)."""
     assert layer and out_md, "--summarize needs --summary-layer and --out-md"
-    sections, fetch, write, dur = [], {}, {}, {}
+    sections, fetch, write, dur, l2 = [], {}, {}, {}, {}
     for d in dirs:
         dbs = [os.path.join(r, f) for r, _, fs in os.walk(d) for f in fs if f.endswith("_results.db")]
         assert dbs, f"no *_results.db under {d}"
@@ -438,6 +438,10 @@ def summarize(dirs, layer, out_md):
                 fetch[n] = a["pmc"]["FETCH_SIZE"] / a["calls"]
             if "WRITE_SIZE" in a["pmc"]:
                 write[n] = a["pmc"]["WRITE_SIZE"] / a["calls"]
+            hit = sum(v for k, v in a["pmc"].items() if k.startswith("TCC_HIT"))
+            miss = sum(v for k, v in a["pmc"].items() if k.startswith("TCC_MISS"))
+            if hit + miss > 0:
+                l2[n] = {"hit_per_call": hit / a["calls"], "miss_per_call": miss / a["calls"], "hit_rate": hit / (hit + miss)}
             if not a["pmc"]:
                 dur[n] = a["ns"] / a["calls"] / 1e3
         sections.append((os.path.basename(os.path.normpath(d)), lines))
@@ -467,6 +471,15 @@ def summarize(dirs, layer, out_md):
         text += [f"## {name}", "", "```"] + lines + ["```", ""]
     text += ["## HBM bytes per launch (FETCH_SIZE x factor + WRITE_SIZE x factor)", "", "```"]
     text += [f"{n:40s} {k['hbm_bytes'] / 1e6:10.1f} MB" for n, k in kernels.items()] + ["```", ""]
+    if l2:
+        # every request that reaches the L2 (TCC) is a hit or a miss there; a miss goes on to the memory-side
+        # cache (MALL) and HBM, which FETCH_SIZE above counts
+        text += ["## L2 (TCC) requests per launch and hit rate (TCC_HIT_sum, TCC_MISS_sum over all channels)", "", "```"]
+        text += [f"{n:40s} hit {v['hit_per_call'] / 1e6:9.2f} M  miss {v['miss_per_call'] / 1e6:9.2f} M  hit rate {100 * v['hit_rate']:5.1f} %"
+                 for n, v in l2.items() if n.startswith("attn_")] + ["```", ""]
+        for n, v in l2.items():
+            if n in kernels:
+                kernels[n]["l2_hit_rate"] = round(v["hit_rate"], 4)
     body = "\n".join(text)
     if os.path.exists(out_md) and "<!-- generated below -->" in open(out_md).read():
         head = open(out_md).read().split("<!-- generated below -->")[0]
