@@ -548,6 +548,26 @@ __device__ __forceinline__ void dq_tile(uint32_t ksm, uint32_t vsm, const TileLa
     // wrel (masked variant only): (first query position of the wavefront) - (first key of the
     // tile); a 32-key half of the tile that no row of the wavefront can see is skipped.
     const int half = lane >> 5;
+    // Masked variant, per lane and tile: key r = rc + 4*half of the tile (rc a compile-time constant per
+    // accumulator register) is visible to the lane's row iff 0 <= dbase - r < wl and r < key_lim, i.e. iff
+    // lo <= rc <= hi with lo = dbase - 4*half - wl + 1 and hi = min(dbase - 4*half, key_lim - 4*half - 1):
+    // (unsigned)(mlo + rc) < width with mlo = -lo, width = max(0, hi - lo + 1).  One add, one compare, one
+    // select per element, and no lane-dependent row index per register to keep alive across the key loop.
+    // (All in wrapping 32-bit arithmetic: dbase of a dead row is about -2^30, wl at most 2^30, so the true
+    // values of mlo + rc and width stay below 2^32 and 2^31.)  For 64-row wavefronts, whose register file
+    // is full; the 32-row instantiations keep the plain form, which costs them no spill.
+    constexpr bool FOLDED = NQB == 2;
+    unsigned mlo[NQB], width[NQB];
+    if (MASKED && FOLDED) {
+#pragma unroll
+        for (int qb = 0; qb < NQB; ++qb) {
+            const int dbh = dbase[qb] - 4 * half;
+            const unsigned lo_ = (unsigned)dbh - wl[qb] + 1u;
+            const int hi_ = min(dbh, key_lim - 4 * half - 1);
+            mlo[qb] = 0u - lo_;
+            width[qb] = (unsigned)max(0, (int)((unsigned)hi_ - lo_ + 1u));
+        }
+    }
 #pragma unroll
     for (int kb = 0; kb < 2; ++kb) {
         if (MASKED && ((32 * kb > wrel + 32 * NQB - 1) || (32 * kb + 31 < wrel - (int)weff + 1) || (32 * kb >= key_lim))) continue;
@@ -574,7 +594,8 @@ __device__ __forceinline__ void dq_tile(uint32_t ksm, uint32_t vsm, const TileLa
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
                 float pe = fast_exp2(fmaf(s[qb][i], c, -lse2[qb]));
-                if (MASKED) {
+                if (MASKED && FOLDED) pe = (mlo[qb] + (unsigned)(32 * kb + 8 * (i >> 2) + (i & 3))) < width[qb] ? pe : 0.0f;
+                if (MASKED && !FOLDED) {
                     const int r = 32 * kb + crow(i, half);
                     const bool vis = ((unsigned)(dbase[qb] - r) < wl[qb]) & (r < key_lim);
                     pe = vis ? pe : 0.0f;
@@ -608,6 +629,11 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_bwd_dq_kernel(co
 
     const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
     const int l32 = lane & 31, half = lane >> 5;
+    // For the cold paths (a tile that sticks out of the tensor, the epilogue): the wave index as a scalar and
+    // the lane index recomputed on the spot, so that nothing derived from them has to survive the key loop
+    // in a register file that is full (64-row wavefronts).
+    const int w_s = __builtin_amdgcn_readfirstlane(w);
+    auto fresh_lane = []() __attribute__((always_inline)) { return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)); };
 
     const int n_hc = (a.r + HPB - 1) / HPB;
     int bid = blockIdx.x;
@@ -728,8 +754,9 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_bwd_dq_kernel(co
             tile_async_inner(smem[stage][0], ktile, klane, w);
             tile_async_inner(smem[stage][1], vtile, vlane, w);
         } else {
-            tile_async(smem[stage][0], kbase, a.ks.s, next_row0, a.Skv, lane, w);
-            tile_async(smem[stage][1], vbase, a.vs.s, next_row0, a.Skv, lane, w);
+            const int fl = fresh_lane();
+            tile_async(smem[stage][0], kbase, a.ks.s, next_row0, a.Skv, fl, w_s);
+            tile_async(smem[stage][1], vbase, a.vs.s, next_row0, a.Skv, fl, w_s);
         }
         ktile += kTile * a.ks.s;
         vtile += kTile * a.vs.s;
@@ -768,12 +795,17 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_bwd_dq_kernel(co
     }
     __syncthreads();
     if (active) {
-        bf16 *stage = reinterpret_cast<bf16 *>(&smem[0][0][0]) + w * 32 * kLS;
+        // wave-uniform quantities recomputed from scalars
+        const int hsel_s = hc * HPB + (w_s % HPB);
+        const int head_s = g * a.r + hsel_s;
+        const int qw0_s = qt * BM + WM * (w_s / HPB);
+        const int fl = fresh_lane();
+        bf16 *stage = reinterpret_cast<bf16 *>(&smem[0][0][0]) + w_s * 32 * kLS;
 #pragma unroll
         for (int qb = 0; qb < NQB; ++qb) {
-            const int r0 = qw0 + 32 * qb;
-            bf16 *row0 = a.dq + (int64_t)b * a.dqs.b + (int64_t)head * a.dqs.h + (int64_t)r0 * a.dqs.s;
-            store_rows32(stage, dq[qb], a.scale, row0, a.dqs.s, a.Sq - r0, lane);
+            const int r0 = qw0_s + 32 * qb;
+            bf16 *row0 = a.dq + (int64_t)b * a.dqs.b + (int64_t)head_s * a.dqs.h + (int64_t)r0 * a.dqs.s;
+            store_rows32(stage, dq[qb], a.scale, row0, a.dqs.s, a.Sq - r0, fl);
             __builtin_amdgcn_wave_barrier();
         }
     }
