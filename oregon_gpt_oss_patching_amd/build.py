@@ -11,10 +11,9 @@ import subprocess
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 SOURCE = os.path.join(_HERE, "csrc", "gptoss_attn.hip")
-LIBRARY = os.environ.get("GPTOSS_LIB_OUT") or os.path.join(_HERE, "libgptoss_attn.so")
+LIBRARY = os.path.join(_HERE, "libgptoss_attn.so")
 
 HIPCC_FLAGS = [
-    *(__import__("os").environ.get("GPTOSS_DEFS", "").split()),
     "--offload-arch=gfx950",
     "-O3",
     "-std=c++17",

@@ -182,15 +182,16 @@ __device__ __forceinline__ int swz(int r) { return (((r >> 1) & 1) << 2) | (((r 
 typedef __attribute__((address_space(3))) void lds_void_t;
 typedef __attribute__((address_space(1))) const void glb_void_t;
 
-// The copy instruction itself, written as inline assembly on purpose.  Issued through the compiler's
-// builtin, every LDS read that follows a copy is made to wait for ALL outstanding copies (the compiler
-// cannot tell which LDS bytes a copy writes, and a workgroup barrier waits for them as well), which
+// The copy instruction written as inline assembly (used by attn_bwd_dkdv64_kernel only).  Issued through
+// the compiler's builtin, every LDS read that follows a copy is made to wait for ALL outstanding copies (the
+// compiler cannot tell which LDS bytes a copy writes, and a workgroup barrier waits for them as well), which
 // turns a three-stage pipeline into "issue, wait for what was just issued, compute".  Hidden in the
-// assembly the copies are invisible to that bookkeeping; ordering is then entirely this code's
+// assembly the copies are invisible to that bookkeeping; ordering is then entirely the kernel's
 // business: wait_vmcnt<N>() before the barrier that hands a stage to its readers, and a barrier
 // between the last read of a stage and the copy that overwrites it.  (Compiler-generated vmcnt waits
 // for its own loads stay correct: loads return in order, so unknown extra loads only make such a wait
-// longer.)  M0 holds the wave-uniform LDS base; nothing else in these kernels uses M0.
+// longer.)  M0 holds the wave-uniform LDS base; nothing else in these kernels uses M0.  The kernels with
+// two wavefronts per SIMD keep the builtin: there the hidden form measured slower.
 // lane L's 16 bytes at gbase + voff land at lds_base + 16 * L
 __device__ __forceinline__ void lds_dma16(uint32_t lds_base, const void *gbase, uint32_t voff) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(voff), "s"(gbase) : "memory");
@@ -202,28 +203,14 @@ __device__ __forceinline__ void lds_dma16_plus(uint32_t lds_base, const void *gb
     if constexpr (IMM == 0) lds_dma16(lds_base, gbase, voff);
     else asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(voff), "s"(gbase), "n"(IMM) : "memory", "scc");
 }
-// the same with a full per-lane address
-__device__ __forceinline__ void lds_dma16_at(uint32_t lds_base, const void *gaddr) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_base), "v"(gaddr) : "memory");
-}
 // lane L's 4 bytes at gbase + voff land at lds_base + 4 * L
 __device__ __forceinline__ void lds_dma4(uint32_t lds_base, const void *gbase, uint32_t voff) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds_base), "v"(voff), "s"(gbase) : "memory");
-}
-// lane L's 4 bytes at gaddr land at lds_base + 4 * L
-__device__ __forceinline__ void lds_dma4_at(uint32_t lds_base, const void *gaddr) {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(lds_base), "v"(gaddr) : "memory");
-}
-__device__ __forceinline__ uint32_t lds_uniform_addr(const void *p) {
-    typedef __attribute__((address_space(3))) char lds_char;
-    return (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(uintptr_t)(lds_char *)p);
 }
 
 // Issues the 4-wavefront asynchronous copy of tile rows [row0, row0+64) (rows at or
 // beyond row_end re-read the last valid row: their products are masked, they only
 // have to be finite).  Each wavefront issues two instructions.
-// HIDDEN: through the inline-assembly copy above (the caller then owns all the ordering).
-template <bool HIDDEN = false>
 __device__ __forceinline__ void tile_async(char *lds_tile, const bf16 *base, int64_t stride_s, int row0,
                                            int row_end, int lane, int w) {
 #pragma unroll
@@ -232,8 +219,7 @@ __device__ __forceinline__ void tile_async(char *lds_tile, const bf16 *base, int
         const int c = (lane & 7) ^ swz(r);
         const int row = min(row0 + r, row_end - 1);
         const bf16 *src = base + (int64_t)row * stride_s + c * 8;
-        if constexpr (HIDDEN) lds_dma16_at(lds_uniform_addr(lds_tile + (16 * w + 8 * k) * kRowBytes), src);
-        else __builtin_amdgcn_global_load_lds((glb_void_t *)src, (lds_void_t *)(lds_tile + (16 * w + 8 * k) * kRowBytes), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((glb_void_t *)src, (lds_void_t *)(lds_tile + (16 * w + 8 * k) * kRowBytes), 16, 0, 0);
     }
 }
 
@@ -256,20 +242,12 @@ __device__ __forceinline__ AsyncLaneOffsets make_async_offsets(int64_t stride_s,
     return o;
 }
 
-template <bool HIDDEN = false>
 __device__ __forceinline__ void tile_async_inner(char *lds_tile, const bf16 *tile, const AsyncLaneOffsets &o, int w) {
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
-        if constexpr (HIDDEN) lds_dma16(lds_uniform_addr(lds_tile + (16 * w + 8 * k) * kRowBytes), tile, o.off[k]);
-        else __builtin_amdgcn_global_load_lds((glb_void_t *)(reinterpret_cast<const char *>(tile) + o.off[k]),
-                                              (lds_void_t *)(lds_tile + (16 * w + 8 * k) * kRowBytes), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((glb_void_t *)(reinterpret_cast<const char *>(tile) + o.off[k]),
+                                         (lds_void_t *)(lds_tile + (16 * w + 8 * k) * kRowBytes), 16, 0, 0);
     }
-}
-// lane L's 4 bytes at gaddr land at lds_dst + 4 * L
-template <bool HIDDEN = false>
-__device__ __forceinline__ void word_async(void *lds_dst, const void *gaddr) {
-    if constexpr (HIDDEN) lds_dma4_at(lds_uniform_addr(lds_dst), gaddr);
-    else __builtin_amdgcn_global_load_lds((glb_void_t *)gaddr, (lds_void_t *)lds_dst, 4, 0, 0);
 }
 
 // Waits until at most `n` of this wavefront's vector-memory operations are outstanding.
