@@ -80,3 +80,25 @@ def test_tiled_packed_rows_match_eager_and_golden(golden_dir):
     got = (o,) + T.tiled_bwd(q, k, v, sinks, o, lse, d_out, SCALE, None, 0, None, ds)[:4]
     for a, b_ in zip(ref, got):
         assert torch.allclose(a.float(), b_, atol=3e-6, rtol=1e-5)
+
+
+def test_three_bf16_terms_carry_an_fp32_number():
+    """The dK/dV kernels take lse / scale and -delta as three bf16 terms each (hi = bf16(x), mid = bf16(x - hi),
+    lo = bf16(x - hi - mid), csrc/attn_common.h split_row_stats) and let the matrix pipe add them up in fp32.
+    The claim the kernels rest on, checked here in torch's own bf16 arithmetic (round to nearest even, as the
+    device's conversion): both residuals are exact in fp32 and the three terms add up to x exactly, for the
+    whole range the statistics live in (logsumexp / scale up to a few thousand, delta of either sign, tiny values)."""
+    import torch
+    gen = torch.Generator().manual_seed(5)
+    mags = torch.tensor([1e-6, 1e-3, 0.1, 1.0, 17.0, 300.0, 4096.0, 1.0e5])
+    x = (torch.randn(8, 20000, generator=gen) * mags.view(8, 1)).reshape(-1).float()
+    x = torch.cat([x, torch.tensor([0.0, -0.0, 1.0, -1.0, 255.5, 65535.99, 2.0 ** -20, 3.0e38 / 2 ** 40])])
+    hi = x.to(torch.bfloat16).float()
+    r1 = x - hi
+    assert torch.equal(r1.double(), x.double() - hi.double())          # the first residual is exact
+    mid = r1.to(torch.bfloat16).float()
+    r2 = r1 - mid
+    assert torch.equal(r2.double(), r1.double() - mid.double())        # so is the second
+    lo = r2.to(torch.bfloat16).float()
+    assert torch.equal(lo, r2)                                         # and it fits 8 mantissa bits: nothing is left
+    assert torch.equal((hi + mid) + lo, x) and torch.equal((lo + mid) + hi, x)
