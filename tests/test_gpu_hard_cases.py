@@ -230,9 +230,12 @@ def test_dkdv64_route_has_the_bits_of_the_32_key_kernel(A, b, h, g, s):
     print(f"case B={b} H={h} G={g} S={s}", flush=True)
     q, k, v, sinks, d_out = (t.to(DEV) for t in E.make_inputs(1700 + s, b, h, g, s, 64, torch.bfloat16))
     o, lse = A.attention_forward(q, k, v, sinks, SCALE, None)
-    one = A.attention_backward(q, k, v, sinks, o, lse, d_out, SCALE, None)
     two = A.attention_backward(q, k, v, sinks, o, lse, d_out, SCALE, None, 0, [s] * b)
-    torch.cuda.synchronize()
-    for name, x, y in zip(("dq", "dk", "dv", "dsinks"), one, two):
-        assert torch.isfinite(x.float()).all(), name
-        assert torch.equal(x, y), name
+    # several runs of the hand-scheduled kernel: its register hazards are handled in the source, not by the
+    # compiler, and a violation would show as bits that change from run to run
+    for rep in range(4):
+        one = A.attention_backward(q, k, v, sinks, o, lse, d_out, SCALE, None)
+        torch.cuda.synchronize()
+        for name, x, y in zip(("dq", "dk", "dv", "dsinks"), one, two):
+            assert torch.isfinite(x.float()).all(), (name, rep)
+            assert torch.equal(x, y), (name, rep)
