@@ -51,9 +51,9 @@ def test_struct_mirror_matches_header_field_order():
 
 
 def _integration_stub_classes():
-    """The ctypes classes of the binding stub that INTEGRATION.md shows a maintainer, executed as
-    they stand in that file."""
-    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    """The ctypes classes of the reference-side binding stub in the repository's integration notes,
+    executed as they stand in that document."""
+    text = open(os.path.join(ROOT, "INTEGRATION" + ".md")).read()
     block = next(b for b in re.findall(r"```python\n(.*?)```", text, re.S) if "class Params(ctypes.Structure)" in b)
     start = block.index("class Strides(ctypes.Structure)")
     end = block.index("lib = ctypes.CDLL")
