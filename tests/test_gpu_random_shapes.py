@@ -11,8 +11,9 @@ What is compared, per case (bf16 tolerances as in test_gpu_parity, fp32 as in te
     comparison is well conditioned for every case of the sweep.  End to end (against autograd through
     the eager oracle) delta = rowsum(dO * O) taken from a bf16-rounded O loses all relative accuracy
     in dQ when every row keeps a single key with probability ~1 (window 1, sink logit far below),
-    and in a dSinks that is the cancelling sum of a few rows; test_gpu_parity holds the end-to-end
-    comparisons on well-conditioned problems.
+    and in a dSinks that is the cancelling sum of a few rows.  test_random_problem_end_to_end below makes that
+    end-to-end comparison for every draw whose rows keep eight keys or more, with dSinks held to the scale of
+    its terms; test_gpu_parity holds the end-to-end comparisons on the regular shapes.
 """
 import random
 
@@ -90,3 +91,64 @@ def test_random_problem(case):
         TF.compare([o, lse, dq, dk, dv, dsk], [ro, rlse, tdq.double(), tdk.double(), tdv.double(), tds.double()])
     else:
         TP.compare_all((o, lse, dq, dk, dv, dsk), (ro, rlse, tdq, tdk, tdv, tds))
+
+
+# ---- the same draws, end to end ----------------------------------------------------------------------
+
+E2E_ATOL = 3e-2
+
+
+def _well_conditioned(c):
+    """End to end (autograd through the eager oracle on the inputs alone) the kernels' delta = rowsum(dO * O)
+    comes from the bf16-rounded O they saved, as the reference's does (attention_kernel.py:119).  That is
+    harmless unless dS = P (dP - delta) is a difference of nearly equal numbers everywhere, which is what a row
+    with one or two visible keys is (window 1 or 2: P ~ 1 on a single key).  Those draws are left to the
+    function-level comparison above."""
+    return c["w"] is None or c["w"] >= 8
+
+
+@pytest.mark.parametrize("case", range(N_CASES))
+def test_random_problem_end_to_end(case):
+    """O, lse, dQ, dK, dV against the eager oracle and its autograd backward on the same inputs, nothing
+    taken from the kernels.  bf16: relative L2 1e-2 and |x - ref| <= 3e-2 + 2^-8 |ref| (2e-2 where |ref| <= 1 is
+    what test_gpu_parity asserts on its regular shapes; the irregular draws here include 8 to 16 heads per
+    KV head on rows of a few dozen keys, where the bf16 rounding of P alone reaches 2.5e-2, see
+    test_gpu_hard_cases).  dSinks, a sum over all rows that may cancel, is held to 1e-2 of the sum of the
+    magnitudes of its terms.  fp32 tensors: the bounds of test_gpu_float32."""
+    import oregon_gpt_oss_patching_amd as A
+    c = draw_case(case)
+    if not _well_conditioned(c):
+        pytest.skip("one or two keys per row: dS is a cancelling difference, compared at function level only")
+    b, sq, w, q_offset, seqlens, dt = c["b"], c["sq"], c["w"], c["q_offset"], c["seqlens"], c["dt"]
+    q, k, v, sinks, d_out = E.make_inputs(5000 + case, b, c["h"], c["g"], sq, 64, dt, skv=c["skv"])
+    sinks = (sinks + c["shift"]).to(dt)
+    if seqlens is not None:
+        d_out = TP.mask_dout(d_out, seqlens)
+    ds = E.doc_start_from_lengths(c["lens"], sq) if c["lens"] is not None else None
+    qd, kd, vd, sd, dod = (t.to(DEV) for t in (q, k, v, sinks, d_out))
+    dsd = ds.to(DEV) if ds is not None else None
+    print(c, flush=True)
+    o, lse = A.attention_forward(qd, kd, vd, sd, TP.SCALE, w, q_offset, seqlens, dsd)
+    dq, dk, dv, dsk = A.attention_backward(qd, kd, vd, sd, o, lse, dod, TP.SCALE, w, q_offset, seqlens, doc_start=dsd)
+    torch.cuda.synchronize()
+    got = [t.cpu() for t in (o, lse, dq, dk, dv, dsk)]
+
+    wide = torch.float64 if dt == torch.float32 else torch.float32
+    f = [t.to(wide) for t in (q, k, v, sinks, d_out)]
+    ro, rdq, rdk, rdv, rds = E.eager_attention_grads(*f, TP.SCALE, w, q_offset, seqlens, ds)
+    rlse = E.logsumexp_rows(f[0], f[1], f[3], TP.SCALE, w, q_offset, seqlens, ds)
+    # dSinks = -sum over rows of exp(sink - lse) * delta (attention_kernel.py:173-176): the scale of its terms
+    p_sink = torch.exp(f[3].view(1, -1, 1).double() - rlse.double())                      # (B, H, S)
+    delta = (f[4].double() * ro.double()).sum(-1).permute(0, 2, 1)                           # (B, H, S)
+    term_sum = (p_sink * delta).abs().sum(dim=(0, 2))                                        # (H,)
+    assert bool(((got[5].double() - rds.double()).abs() <= 1e-2 * term_sum + 1e-6).all()), "dsinks"
+    if dt == torch.float32:
+        TF.compare(got[:5] + [rds.float()], [ro, rlse, rdq, rdk, rdv, rds])
+        return
+    TP.check("o", got[0], ro)
+    assert float((got[1] - rlse.float()).abs().max()) <= TP.LSE_TOL
+    for name, x, r in (("dq", got[2], rdq), ("dk", got[3], rdk), ("dv", got[4], rdv)):
+        x, r = x.float(), r.float()
+        assert TP.rel_l2(x, r) <= 1e-2, (name, TP.rel_l2(x, r))
+        err = (x - r).abs()
+        assert bool((err <= E2E_ATOL + 2.0 ** -8 * r.abs()).all()), (name, float(err.max()), float(r.abs().max()))
