@@ -54,17 +54,25 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv64_kernel(const KArgs a) 
     int bid = blockIdx.x;
     const int g = bid % a.G; bid /= a.G;
     const int b = bid % a.B; bid /= a.B;
+    const int part = bid % a.dkdv_parts; bid /= a.dkdv_parts;
     const int kt = bid;                                   // ascending: most work first
     const int j0 = kt * BN;                               // first key of the workgroup
     const int wj0 = j0 + WK * w;                          // first key of the wavefront
 
-    // The workgroup walks the query tiles from the last one down to the one that holds its first key, all
-    // heads of the group per tile.  Wavefront w's diagonal tile is w tiles above the end of the walk.
-    const int qt_hi = a.Sq / kTile, qt_lo = j0 / kTile;
-    const int n_it = (qt_hi - qt_lo) * a.r;
+    // The query tiles that can see the workgroup's keys run from the one that holds its first key to the
+    // last one; with dkdv_parts > 1 they are cut into that many consecutive slices, one per workgroup, each
+    // of which leaves an fp32 partial sum (attn_bwd_dkdv_reduce_kernel adds them in slice order).  The
+    // workgroup walks its slice from the last tile down, all heads of the group per tile.  Wavefront w's
+    // diagonal tile is tile wq; above it every tile is interior, below it none concerns the wavefront.
+    const int qt_all_hi = a.Sq / kTile, qt_lo = j0 / kTile;
+    const int nq_all = qt_all_hi - qt_lo;
+    const int slice = (nq_all + a.dkdv_parts - 1) / a.dkdv_parts;
+    const int qt_hi = qt_all_hi - part * slice;                       // end of this workgroup's slice
+    const int nq = max(0, min(slice, nq_all - part * slice));
+    const int n_it = nq * a.r;
     const int wq = qt_lo + w;                             // the query tile on the wavefront's diagonal
-    const int n_int = wq < qt_hi ? (qt_hi - 1 - wq) * a.r : 0;     // iterations on interior tiles
-    const int n_mask = wq < qt_hi ? a.r : 0;                       // then on the diagonal tile
+    const int n_int = (wq < qt_all_hi ? max(0, min(nq, qt_hi - 1 - wq)) : 0) * a.r;          // iterations on interior tiles
+    const int n_mask = (wq < qt_hi && wq >= qt_hi - nq) ? a.r : 0;                            // then on the diagonal tile
 
     // K, V fragments (B operands): lane = key, slots = head_dim
     bf16x8 kf[NB][4], vf[NB][4];
@@ -128,7 +136,7 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv64_kernel(const KArgs a) 
     const uint32_t stat_voff = w * (C::kWaveRows * 16) + lane * 4;
     const uint32_t stat_dst = __builtin_amdgcn_readfirstlane(C::kStatOff - w * (C::kWaveRows * kRowBytes) + w * (C::kWaveRows * 16));
     int iss_h = 0, iss_left = n_it;
-    const int i0_first = (qt_hi - 1) * kTile;
+    const int i0_first = max(qt_hi - 1, 0) * kTile;      // (an empty slice requests nothing: n_it is 0)
     const bf16 *qtile = a.q + (int64_t)b * a.qs.b + (int64_t)(g * a.r) * a.qs.h + (int64_t)i0_first * a.qs.s;
     const bf16 *gtile = a.d_o + (int64_t)b * a.dos.b + (int64_t)(g * a.r) * a.dos.h + (int64_t)i0_first * a.dos.s;
     const u32x4 *stat_src = a.split + ((int64_t)b * a.H + (int64_t)g * a.r) * a.Sq + i0_first;     // wave-uniform
@@ -370,6 +378,31 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv64_kernel(const KArgs a) 
 
     wait_vmcnt<0>();          // the repeated copies of the last requests
     agpr_accumulators_settled(dk, dv);
+    if (a.dkdv_parts > 1) {
+        // unscaled fp32 partial sums; lane = key row, register i of block dblk = column 32*dblk + crow(i, half),
+        // four consecutive columns per 16-byte store
+        const int64_t tensor = (int64_t)a.B * a.G * a.Skv * kD;
+        float *pk = a.dkdv_partial + (int64_t)part * 2 * tensor + (((int64_t)b * a.G + g) * a.Skv) * kD;
+        float *pv = pk + tensor;
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            const int j = wj0 + 32 * nb + l32;
+            if (j < a.Skv) {
+#pragma unroll
+                for (int dblk = 0; dblk < 2; ++dblk)
+#pragma unroll
+                    for (int a4 = 0; a4 < 4; ++a4) {
+                        const int col = 32 * dblk + 8 * a4 + 4 * half;
+                        f32x4 xk, xv;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) { xk[e] = dk[nb][dblk][4 * a4 + e]; xv[e] = dv[nb][dblk][4 * a4 + e]; }
+                        *reinterpret_cast<f32x4 *>(pk + (int64_t)j * kD + col) = xk;
+                        *reinterpret_cast<f32x4 *>(pv + (int64_t)j * kD + col) = xv;
+                    }
+            }
+        }
+        return;
+    }
     __syncthreads();
     bf16 *stage_out = reinterpret_cast<bf16 *>(&smem[0]) + w * 32 * kLS;
 #pragma unroll

@@ -110,14 +110,16 @@ int dkdv_parts_for(const gptoss_attn_params *p) {
     return parts < 1 ? 1 : parts;
 }
 
-// Long full-causal self-attention rows go to attn_bwd_dkdv64_kernel (64 keys per wavefront, one wavefront
-// per SIMD): bf16, no window, no padded or packed rows, no offset, Sq == Skv a multiple of 64, and enough
-// key blocks that the 32-key kernel would not cut them into slices (then the 256-key workgroups of the
-// 64-key kernel are at least 257, one per compute unit and more).  Same bits as the 32-key kernel.
-bool dkdv64_route(const gptoss_attn_params *p) {
+// Full-causal self-attention goes to attn_bwd_dkdv64_kernel (64 keys per wavefront, one wavefront per SIMD)
+// when the shape is the one it is written for (bf16, no window, no padded or packed rows, no offset,
+// Sq == Skv a multiple of 64) and there is enough of it: more than 512 key blocks of 128 (then key blocks are
+// whole: at least 257 workgroups of 256 keys, and the same bits as the 32-key kernel), or rows of 2048 keys
+// or more that the host cuts into `parts` slices anyway (the same number of slices as the 32-key kernel
+// would get, so the scratch is the same; -15 % at S = 2048 ... 8192).
+bool dkdv64_route(const gptoss_attn_params *p, int parts) {
     const int64_t blocks = (int64_t)p->G * p->B * ((p->Skv + kDkdvKeys - 1) / kDkdvKeys);
     return p->dtype == GPTOSS_ATTN_BF16 && effective_window(p) == 0 && !p->seqlens && !p->doc_start && p->q_offset == 0 &&
-           !p->q_offset_dev && p->Sq == p->Skv && p->Sq % kTile == 0 && blocks > 512;
+           !p->q_offset_dev && p->Sq == p->Skv && p->Sq % kTile == 0 && (blocks > 512 || (parts > 1 && p->Skv >= 2048));
 }
 
 // workgroups of four independent wavefronts for the float32 kernels
@@ -344,9 +346,13 @@ static int launch_dkdv(const gptoss_attn_params *p, void *stream, bool whole_blo
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (p->dtype == GPTOSS_ATTN_FP32)
         return launch(attn_f32_dkdv_kernel, f32_grid((int64_t)a.B * a.G * ((a.Skv + 31) / 32)), 256, st, a);
-    if (dkdv64_route(p)) return launch(attn_bwd_dkdv64_kernel, (int64_t)a.G * a.B * ((a.Skv + Dkdv64::BN - 1) / Dkdv64::BN), 256, st, a);
     a.dkdv_parts = whole_blocks ? 1 : dkdv_parts_for(p);
     a.dkdv_partial = reinterpret_cast<float *>(reinterpret_cast<char *>(p->delta) + stats_bytes(p));
+    if (dkdv64_route(p, a.dkdv_parts)) {
+        const int s = launch(attn_bwd_dkdv64_kernel, (int64_t)a.G * a.B * a.dkdv_parts * ((a.Skv + Dkdv64::BN - 1) / Dkdv64::BN), 256, st, a);
+        if (s || a.dkdv_parts == 1) return s;
+        return launch(attn_bwd_dkdv_reduce_kernel, ((int64_t)2 * a.B * a.G * a.Skv * 8 + 255) / 256, 256, st, a);
+    }
     const int64_t grid = (int64_t)a.G * a.B * a.dkdv_parts * ((a.Skv + kDkdvKeys - 1) / kDkdvKeys);
     const int s = a.doc_start ? launch(attn_bwd_dkdv_kernel<kDkdvWaves, kDkdvNB, true>, grid, 64 * kDkdvWaves, st, a)
                               : launch(attn_bwd_dkdv_kernel<kDkdvWaves, kDkdvNB, false>, grid, 64 * kDkdvWaves, st, a);

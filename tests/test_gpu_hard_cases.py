@@ -191,9 +191,10 @@ def test_sweep_misses_are_the_bf16_rounding_of_p(A, seed, b, h, g, s, w, atol):
 
 
 # ---- the 64-key dK/dV kernel (long full-causal rows) ------------------------------------------------
-# gptoss_attn_bwd sends bf16 full-causal self-attention without padded or packed rows, Sq a multiple of 64
-# and more than 512 key blocks of 128 to attn_bwd_dkdv64_kernel.  Many short batch rows reach that route
-# at sizes the CPU oracle still handles.
+# gptoss_attn_bwd sends bf16 full-causal self-attention without padded or packed rows and with Sq a multiple
+# of 64 to attn_bwd_dkdv64_kernel when there are more than 512 key blocks of 128 (whole key blocks per
+# workgroup) or, cut into slices, when a row has 2048 keys or more.  Many short batch rows reach the first
+# route at sizes the CPU oracle still handles.
 
 DKDV64_CASES = [
     # B, H, G, S
@@ -220,6 +221,38 @@ def test_dkdv64_route_vs_eager_oracle(A, b, h, g, s):
         TP.compare_all((o[i:i + 1], lse[i:i + 1], dq[i:i + 1], dk[i:i + 1], dv[i:i + 1], rds_i), (ro, rlse, rdq, rdk, rdv, rds_i))
         rds += rds_i.double()
     TP.check("dsinks", ds, rds.float(), atol=None)
+
+
+@pytest.mark.parametrize("b,h,g,s", [
+    (1, 16, 2, 2048),      # 32 key blocks: eight slices of four query tiles per 256-key workgroup
+    (2, 8, 8, 2304),       # 36 tiles, three slices; the last workgroup of a row holds 256 of its 2304 keys
+    (1, 8, 1, 4160),       # S = 16 * 256 + 64: one live wavefront in the last workgroup, eight slices
+    (3, 12, 4, 2112),      # three heads per KV head, S = 8 * 256 + 64
+])
+def test_dkdv64_route_cut_into_slices_vs_eager_oracle(A, b, h, g, s):
+    """Rows of 2048 keys or more with too few key blocks to fill the GPU: the 64-key kernel takes them with
+    every key block's query tiles cut into slices (fp32 partial sums, added in slice order)."""
+    from oregon_gpt_oss_patching_amd import _lib
+    import ctypes
+    from oregon_gpt_oss_patching_amd import attention_kernel as ak
+    print(f"case B={b} H={h} G={g} S={s}", flush=True)
+    inp = E.make_inputs(1900 + s + b, b, h, g, s, 64, torch.bfloat16)
+    # the library cuts this problem: its scratch is larger than the row statistics
+    qd, kd = inp[0].to(DEV), inp[1].to(DEV)
+    p = ak._base_params(qd, kd, kd, None, None, SCALE, 0, 0)
+    assert _lib.load().gptoss_attn_workspace_bytes(ctypes.byref(p)) > 24 * b * h * s + 16 and s >= 2048 and s % 64 == 0
+    got = TP.run_hip(A, *inp, None)
+    o, lse, dq, dk, dv, ds = (t.detach().cpu() for t in got)
+    rds = torch.zeros(h, dtype=torch.float64)
+    for i in range(b):
+        one = [t[i:i + 1] for t in (inp[0], inp[1], inp[2])] + [inp[3], inp[4][i:i + 1]]
+        ro, rlse, rdq, rdk, rdv, rds_i = TP.oracle_eager(*one, None)
+        TP.compare_all((o[i:i + 1], lse[i:i + 1], dq[i:i + 1], dk[i:i + 1], dv[i:i + 1], rds_i), (ro, rlse, rdq, rdk, rdv, rds_i))
+        rds += rds_i.double()
+    TP.check("dsinks", ds, rds.float(), atol=None)
+    again = TP.run_hip(A, *inp, None)
+    for x, y in zip(got, again):
+        assert torch.equal(x, y)          # fixed summation order: the same bits on every run
 
 
 @pytest.mark.parametrize("b,h,g,s", [(1, 64, 8, 16384), (3, 16, 8, 8192 + 64), (16, 8, 4, 1088)])

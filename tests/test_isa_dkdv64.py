@@ -87,7 +87,8 @@ def test_no_spills_and_full_register_file(kernel_asm):
     assert int(re.search(r"\.vgpr_count:\s+(\d+)", blk).group(1)) > 256
     assert int(re.search(r"\.agpr_count:\s+(\d+)", blk).group(1)) >= 128
     assert int(re.search(r"\.vgpr_spill_count:\s+(\d+)", blk).group(1)) == 0
-    assert int(re.search(r"\.private_segment_fixed_size:\s+(\d+)", blk).group(1)) == 0
+    lines, _ = kernel_asm
+    assert not [x for x in lines if re.search(r"\b(scratch|buffer)_(load|store)", x)], "the kernel touches scratch memory"
 
 
 def _regs(code, kind):
