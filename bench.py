@@ -10,8 +10,11 @@ timed as extra keys.
 
 Prints ONE JSON line.  `value` is algorithmic TFLOP/s of fwd+bwd
 (FLOPs = 14 * D * pairs * B * H, pairs = S(S+1)/2), `roofline` describes the
-dominant kernel, `cpu_baseline` is the eager fp32 restatement timed on the host
-cores on a bounded sample of the same workload.
+dominant kernel, `mfma_ceiling` is what a loop of nothing but MFMAs sustains on
+this box on N(0,1) operands and on zeros (the power limit makes the two differ)
+with the MFMA work the kernels execute per second beside it, `cpu_baseline` is
+the eager fp32 restatement timed on the host cores on a bounded sample of the
+same workload.
 
 Two more modes serve the committed profiles:
   --layers full|window   run one layer type only (what rocprofv3 is pointed at)
@@ -300,9 +303,54 @@ def main():
                      "traffic": recorded_traffic("attn_bwd_dkdv64_kernel", "full") if S == 16384 else None},
     }
 
+    # What the matrix pipes sustain on this box under the power limit: a loop of nothing but MFMAs (the library's
+    # measurement aid), on N(0,1) bf16 operands as the attention kernels see them and on zeros.  Beside it the MFMA
+    # work the three kernels execute per second (the dQ kernel recomputes S and dP, the dK/dV kernel adds its
+    # statistics steps: 9 GEMM units + 9.7 % of 4 where 7 are counted).
+    ceiling = mfma_ceiling(stream, sptr)
+    ceiling["executed_tflops"] = {
+        "fwd": round(2 * unit / (kern["full.fwd"] * 1e-3) / 1e12, 1),
+        "dq": round(3 * unit / (kern["full.bwd_dq"] * 1e-3) / 1e12, 1),
+        "dkdv": round(4 * 1.097 * unit / (dkdv_ms * 1e-3) / 1e12, 1),
+        "step": round((9 + 4 * 0.097) * unit / (ms_full * 1e-3) / 1e12, 1)}
+    out["mfma_ceiling"] = ceiling
+
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(args.cpu_seq, D, 0.125)
     print(json.dumps(out))
+
+
+def mfma_ceiling(stream, sptr, iters=6000, reps=20, warm=40):
+    """TFLOP/s of the bare MFMA loop (gptoss_attn_mfma_rate_probe) on N(0,1) bf16 operands and on zeros.  Each
+    variant runs back to back for about a quarter of a second (the clock under the power limit settles over
+    tens of milliseconds); the last `reps` launches are timed."""
+    import torch
+    from oregon_gpt_oss_patching_amd import _lib
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    sink = torch.empty(512 * cus, dtype=torch.float32, device=dev)
+    gen = torch.Generator(device="cpu").manual_seed(11)
+    res = {"kernel": "loop of v_mfma_f32_32x32x16_bf16 only, two wavefronts per SIMD, operands in registers"}
+    for tag, ops in (("n01", torch.randn(1 << 20, generator=gen).to(torch.bfloat16).to(dev)),
+                     ("zeros", torch.zeros(1 << 20, dtype=torch.bfloat16, device=dev))):
+        def launch():
+            n = lib.gptoss_attn_mfma_rate_probe(ops.data_ptr(), ops.numel() * 2, iters, sink.data_ptr(), sink.numel(), sptr)
+            assert n > 0, n
+            return n
+        for _ in range(warm):
+            launch()
+        evs = []
+        for _ in range(reps):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            n = launch()
+            e1.record(stream)
+            evs.append((e0, e1))
+        torch.cuda.synchronize()
+        ms = statistics.median(a.elapsed_time(b) for a, b in evs)
+        res[f"{tag}_tflops"] = round(n * 32768.0 / (ms * 1e-3) / 1e12, 1)
+    return res
 
 
 def config5():

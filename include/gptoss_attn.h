@@ -226,6 +226,20 @@ int gptoss_attn_bwd_static(const gptoss_attn_params *params, void *stream);
 size_t gptoss_attn_static_scratch_bytes(void);
 
 /*
+ * Measurement aid with no counterpart in the reference and no part in the attention path: launches a
+ * loop of nothing but bf16 MFMAs (v_mfma_f32_32x32x16_bf16, two wavefronts per SIMD on every compute
+ * unit, `iters` passes of 16 MFMAs per wavefront) whose operands are read once from `operands`
+ * (`operand_bytes` >= 16, 16-byte aligned device memory, reused cyclically).  A benchmark times it on the
+ * kind of data the attention kernels see to learn what the matrix pipes sustain under the part's power
+ * limit (the clock under such a loop depends on how many operand bits toggle).  `sink` receives one float
+ * per thread (at least 512 * compute units floats, `sink_floats` says how many there are).  Returns the
+ * number of MFMA instructions the launch executes (each 32*32*16*2 FLOP), or a negative value: a
+ * GPTOSS_ATTN_ERR_* code for bad arguments, -1000 - hipError_t for a failed launch.
+ */
+int64_t gptoss_attn_mfma_rate_probe(const void *operands, size_t operand_bytes, int iters, float *sink, size_t sink_floats,
+                                    void *stream);
+
+/*
  * Host-only argument check used by every entry point; `need_bwd` != 0 also
  * requires the backward tensors.  Callable without a GPU.
  */

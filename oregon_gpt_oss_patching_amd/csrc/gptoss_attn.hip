@@ -13,6 +13,7 @@
 #include "attn_common.h"
 #include "attn_f32.h"
 #include "attn_fwd.h"
+#include "mfma_rate.h"
 
 using namespace gptoss;
 
@@ -449,6 +450,21 @@ int gptoss_attn_bwd_static(const gptoss_attn_params *p, void *stream) {
     rc = static_scratch(&q.delta);
     if (rc) return rc;
     return bwd_all(&q, stream, true);
+}
+
+// ---- measurement aid (mfma_rate.h) -----------------------------------------------------------
+int64_t gptoss_attn_mfma_rate_probe(const void *operands, size_t operand_bytes, int iters, float *sink, size_t sink_floats,
+                                    void *stream) {
+    if (!operands || !sink || operand_bytes < 16 || iters <= 0 || !aligned16(operands)) return GPTOSS_ATTN_ERR_NULL_TENSOR;
+    const int64_t blocks = (int64_t)2 * compute_units();       // two workgroups of four wavefronts per compute unit
+    if ((size_t)blocks * 256 > sink_floats || operand_bytes / 16 > 0xffffffffu) return GPTOSS_ATTN_ERR_SHAPE;
+    const u32x4 *ops = static_cast<const u32x4 *>(operands);
+    uint32_t n_vec = (uint32_t)(operand_bytes / 16);
+    void *args[] = {&ops, &n_vec, &iters, &sink};
+    const hipError_t e = hipLaunchKernel(reinterpret_cast<const void *>(mfma_rate_kernel), dim3((unsigned)blocks), dim3(256), args, 0,
+                                         static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return -static_cast<int64_t>(e) - 1000;
+    return blocks * 4 * (int64_t)iters * kMfmaRatePerIter;      // MFMA instructions the launch executes
 }
 
 }  // extern "C"

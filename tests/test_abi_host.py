@@ -232,3 +232,12 @@ def test_workspace_bytes():
     p.Sq = 0
     assert lib.gptoss_attn_workspace_bytes(ctypes.byref(p)) == 0
     assert lib.gptoss_attn_workspace_bytes(None) == 0
+
+
+def test_mfma_rate_probe_refuses_bad_arguments_on_the_host():
+    """The measurement aid checks its arguments before it launches anything."""
+    lib = _lib.load()
+    assert lib.gptoss_attn_mfma_rate_probe(None, 1024, 10, None, 0, None) < 0
+    assert lib.gptoss_attn_mfma_rate_probe(ctypes.c_void_p(256), 8, 10, ctypes.c_void_p(256), 1 << 30, None) < 0     # under 16 bytes
+    assert lib.gptoss_attn_mfma_rate_probe(ctypes.c_void_p(264), 1024, 10, ctypes.c_void_p(256), 1 << 30, None) < 0  # misaligned
+    assert lib.gptoss_attn_mfma_rate_probe(ctypes.c_void_p(256), 1024, 0, ctypes.c_void_p(256), 1 << 30, None) < 0   # no passes

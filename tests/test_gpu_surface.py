@@ -352,3 +352,20 @@ def test_hip_graph_replays_follow_a_query_offset_in_device_memory():
             ref = (o_ref, lse_ref) + tuple(A.attention_backward(q, k, v, sinks, o_ref, lse_ref, d_out, 0.125, window, start))
             for got, want in zip(outs, ref):
                 assert torch.equal(got, want), start
+
+
+def test_mfma_rate_probe_runs_and_counts_its_mfmas():
+    """The measurement aid bench.py uses: launches, returns the number of MFMA instructions it executes
+    (two workgroups of four wavefronts per compute unit, 16 MFMAs per pass) and leaves finite sums."""
+    import ctypes
+    from oregon_gpt_oss_patching_amd import _lib
+    lib = _lib.load()
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    ops = torch.randn(4096, device="cuda").to(torch.bfloat16)
+    sink = torch.full((512 * cus,), float("nan"), dtype=torch.float32, device="cuda")
+    n = lib.gptoss_attn_mfma_rate_probe(ops.data_ptr(), ops.numel() * 2, 50, sink.data_ptr(), sink.numel(),
+                                        torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert n == 2 * cus * 4 * 50 * 16
+    assert bool(torch.isfinite(sink).all())
+    assert lib.gptoss_attn_mfma_rate_probe(ops.data_ptr(), ops.numel() * 2, 50, sink.data_ptr(), 100, None) < 0   # sink too small
