@@ -25,9 +25,10 @@
 //   boundary costs no drain: M1 of the next tile's first substep is issued in the current tile's
 //   last slot.
 //
-// The host sends only problems in which every wavefront meets, in walk order, interior tiles, then the
-// query tile on its diagonal (masked), then tiles it has nothing to do with: bf16, full causal,
-// Sq == Skv a multiple of 64, no offset, no padded or packed rows, key blocks not cut into slices.
+// The host sends only problems in which every wavefront meets, in walk order, at most one tile whose last
+// rows are padding (masked), interior tiles, the query tile on its diagonal (masked), then tiles it has
+// nothing to do with: bf16, full causal, Sq == Skv a multiple of 64, no offset, no packed rows; right-padded
+// batch rows (seqlens) are fine.
 #pragma once
 #include "attn_bwd.h"
 
@@ -43,6 +44,7 @@ struct Dkdv64 {
     static constexpr int kWaveRows = 16;                           // rows of each tile one wavefront copies
 };
 
+template <bool PADDED>          // PADDED: right-padded batch rows (seqlens given)
 __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv64_kernel(const KArgs a) {
     using C = Dkdv64;
     constexpr int NS = C::NS, WK = C::WK, BN = C::BN, NB = 2;
@@ -64,15 +66,23 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv64_kernel(const KArgs a) 
     // of which leaves an fp32 partial sum (attn_bwd_dkdv_reduce_kernel adds them in slice order).  The
     // workgroup walks its slice from the last tile down, all heads of the group per tile.  Wavefront w's
     // diagonal tile is tile wq; above it every tile is interior, below it none concerns the wavefront.
-    const int qt_all_hi = a.Sq / kTile, qt_lo = j0 / kTile;
-    const int nq_all = qt_all_hi - qt_lo;
+    // A right-padded batch row is a shorter row: rows and keys from len on do not exist.  Its last tile may be
+    // partial (len not a multiple of 64): that one goes through the masked body before the interior tiles.
+    const int len = PADDED ? max(0, min(a.Sq, a.seqlens[b])) : a.Sq;
+    const int qt_all_hi = (len + kTile - 1) / kTile, qt_lo = j0 / kTile;
+    const int nq_all = max(0, qt_all_hi - qt_lo);
     const int slice = (nq_all + a.dkdv_parts - 1) / a.dkdv_parts;
     const int qt_hi = qt_all_hi - part * slice;                       // end of this workgroup's slice
     const int nq = max(0, min(slice, nq_all - part * slice));
     const int n_it = nq * a.r;
     const int wq = qt_lo + w;                             // the query tile on the wavefront's diagonal
-    const int n_int = (wq < qt_all_hi ? max(0, min(nq, qt_hi - 1 - wq)) : 0) * a.r;          // iterations on interior tiles
-    const int n_mask = (wq < qt_hi && wq >= qt_hi - nq) ? a.r : 0;                            // then on the diagonal tile
+    const bool wave_live = wj0 < len;                     // (then wq < qt_all_hi)
+    const int t_part = (len % kTile) ? qt_all_hi - 1 : -1;            // the partial tile, if there is one
+    // in walk order: the partial tile if it is in this slice and above the diagonal, the interior tiles, the diagonal tile
+    const bool top_here = PADDED && wave_live && t_part > wq && t_part == qt_hi - 1 && nq > 0;
+    const int n_top = top_here ? a.r : 0;
+    const int n_int = (wave_live ? max(0, min(nq, qt_hi - 1 - wq)) : 0) * a.r - n_top;
+    const int n_mask = (wave_live && wq < qt_hi && wq >= qt_hi - nq) ? a.r : 0;
 
     // K, V fragments (B operands): lane = key, slots = head_dim
     bf16x8 kf[NB][4], vf[NB][4];
@@ -231,10 +241,13 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv64_kernel(const KArgs a) 
     // another one of the same step: the scaled logit of element i (S arrives with lse / scale already
     // taken off), the exponential of element i - 1, the product of element i - 2 and the packing of the
     // pair it completes.
-    // MASKED (the diagonal tile): pair (row r of the tile, the lane's key of block nb) is visible iff
-    // r >= 32 * nb + l32, folded per lane into (unsigned)(mdb[nb] + rc) < mwd[nb] with rc the compile-time
-    // part of the row index (one add, one compare, one select per element, on the logit: an invisible pair
-    // gets -inf and so P = dS = 0).
+    // MASKED (the diagonal tile, a partial last tile): pair (row r of the tile, the lane's key j of block nb) is
+    // visible iff 0 <= dbase + r and r < row_lim, with dbase = (first position of the tile) - j, or hugely
+    // negative for a key that does not exist; folded per lane and tile into (unsigned)(mdb[nb] + rc) < mwd[nb]
+    // with rc the compile-time part of the row index (one add, one compare, one select per element, on the
+    // logit: an invisible pair gets -inf and so P = dS = 0).
+    // (Without padded rows only the diagonal tile is masked, every key exists and every row too: the two numbers
+    // are constants of the lane, set here once.)
     int mdb[NB];
     unsigned mwd[NB];
 #pragma unroll
@@ -242,6 +255,16 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv64_kernel(const KArgs a) 
         mdb[nb] = 4 * half - (32 * nb + l32);
         mwd[nb] = (unsigned)(kTile - (32 * nb + l32));
     }
+    auto set_mask = [&](int tile) __attribute__((always_inline)) {
+        const int pos0 = tile * kTile, row_lim = min(kTile, len - pos0);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            const int j = wj0 + 32 * nb + l32;
+            const int dbase = j < len ? pos0 - j : -0x40000000;
+            mdb[nb] = dbase + 4 * half;
+            mwd[nb] = (unsigned)max(0, mdb[nb] + row_lim - 4 * half);
+        }
+    };
     auto vstep = [&](auto masked_, int t, int i) __attribute__((always_inline)) {
         constexpr bool MASKED = decltype(masked_)::value;
         const int qb = t >> 1, nb = t & 1;
@@ -327,7 +350,7 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv64_kernel(const KArgs a) 
         rotate();
     };
 
-    if (n_int + n_mask > 0) {
+    if (n_top + n_int + n_mask > 0) {
         {   // fill: block 0 of the first tile, M1(0).  The first slot of the loop also issues M2 of "the tile
             // before": for the first tile that is a product of zeros (exact: the accumulators keep their
             // bits), which keeps the loop body free of variants.
@@ -357,10 +380,24 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv64_kernel(const KArgs a) 
         // (The explicit waits in front of the loops: whatever loads the compiler itself has in flight here,
         // reloads of spilled registers included, are then known to have arrived, and it puts no vmcnt wait of
         // its own into the loops, where it would drain the copies in flight on every pass.)
-        wait_vmcnt<0>();
-        for (int it = 0; it < n_int; ++it) body(F{});
-        wait_vmcnt<0>();
-        for (int it = 0; it < n_mask; ++it) body(T{});
+        if constexpr (PADDED) {
+            // two phases of the same two loops, masked then interior: the partial tile and the interior tiles,
+            // then the diagonal tile and nothing
+#pragma unroll 1
+            for (int ph = 0; ph < 2; ++ph) {
+                const int nm = ph == 0 ? n_top : n_mask, ni = ph == 0 ? n_int : 0;
+                set_mask(ph == 0 ? t_part : wq);
+                wait_vmcnt<0>();
+                for (int it = 0; it < nm; ++it) body(T{});
+                wait_vmcnt<0>();
+                for (int it = 0; it < ni; ++it) body(F{});
+            }
+        } else {
+            wait_vmcnt<0>();
+            for (int it = 0; it < n_int; ++it) body(F{});
+            wait_vmcnt<0>();
+            for (int it = 0; it < n_mask; ++it) body(T{});
+        }
         // drain: M2(3)
         GPTOSS_FENCE();
 #pragma unroll
@@ -369,7 +406,7 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv64_kernel(const KArgs a) 
     }
     // ---- the rest of the walk: nothing to compute, but every wavefront keeps the workgroup's rhythm of
     // barriers and requests ----
-    for (int k = n_int + n_mask; k < n_it; ++k) {
+    for (int k = n_top + n_int + n_mask; k < n_it; ++k) {
         arrive();
         issue(c0);
         rotate();

@@ -112,14 +112,14 @@ int dkdv_parts_for(const gptoss_attn_params *p) {
 }
 
 // Full-causal self-attention goes to attn_bwd_dkdv64_kernel (64 keys per wavefront, one wavefront per SIMD)
-// when the shape is the one it is written for (bf16, no window, no padded or packed rows, no offset,
-// Sq == Skv a multiple of 64) and there is enough of it: more than 512 key blocks of 128 (then key blocks are
+// when the shape is the one it is written for (bf16, no window, no packed rows, no offset, Sq == Skv a
+// multiple of 64; right-padded batch rows are fine) and there is enough of it: more than 512 key blocks of 128 (then key blocks are
 // whole: at least 257 workgroups of 256 keys, and the same bits as the 32-key kernel), or rows of 2048 keys
 // or more that the host cuts into `parts` slices anyway (the same number of slices as the 32-key kernel
 // would get, so the scratch is the same; -15 % at S = 2048 ... 8192).
 bool dkdv64_route(const gptoss_attn_params *p, int parts) {
     const int64_t blocks = (int64_t)p->G * p->B * ((p->Skv + kDkdvKeys - 1) / kDkdvKeys);
-    return p->dtype == GPTOSS_ATTN_BF16 && effective_window(p) == 0 && !p->seqlens && !p->doc_start && p->q_offset == 0 &&
+    return p->dtype == GPTOSS_ATTN_BF16 && effective_window(p) == 0 && !p->doc_start && p->q_offset == 0 &&
            !p->q_offset_dev && p->Sq == p->Skv && p->Sq % kTile == 0 && (blocks > 512 || (parts > 1 && p->Skv >= 2048));
 }
 
@@ -350,7 +350,8 @@ static int launch_dkdv(const gptoss_attn_params *p, void *stream, bool whole_blo
     a.dkdv_parts = whole_blocks ? 1 : dkdv_parts_for(p);
     a.dkdv_partial = reinterpret_cast<float *>(reinterpret_cast<char *>(p->delta) + stats_bytes(p));
     if (dkdv64_route(p, a.dkdv_parts)) {
-        const int s = launch(attn_bwd_dkdv64_kernel, (int64_t)a.G * a.B * a.dkdv_parts * ((a.Skv + Dkdv64::BN - 1) / Dkdv64::BN), 256, st, a);
+        const int64_t grid64 = (int64_t)a.G * a.B * a.dkdv_parts * ((a.Skv + Dkdv64::BN - 1) / Dkdv64::BN);
+        const int s = a.seqlens ? launch(attn_bwd_dkdv64_kernel<true>, grid64, 256, st, a) : launch(attn_bwd_dkdv64_kernel<false>, grid64, 256, st, a);
         if (s || a.dkdv_parts == 1) return s;
         return launch(attn_bwd_dkdv_reduce_kernel, ((int64_t)2 * a.B * a.G * a.Skv * 8 + 255) / 256, 256, st, a);
     }

@@ -223,6 +223,39 @@ def test_dkdv64_route_vs_eager_oracle(A, b, h, g, s):
     TP.check("dsinks", ds, rds.float(), atol=None)
 
 
+@pytest.mark.parametrize("b,h,g,s,lens", [
+    (17, 8, 4, 1024, [1024, 1, 63, 64, 65, 127, 128, 129, 255, 256, 257, 500, 512, 640, 703, 960, 1023]),
+    (16, 8, 4, 1088, [1088, 1087, 1025, 1024, 1023, 961, 960, 959, 897, 832, 769, 700, 320, 193, 64, 2]),
+    (2, 16, 2, 2304, [2304, 1531]),        # cut into slices: the partial tile sits in the first slice only
+    (3, 8, 8, 2112, [2049, 2112, 70]),
+])
+def test_dkdv64_route_right_padded_rows(A, b, h, g, s, lens):
+    """Right-padded batch rows on the 64-key route: lengths on, one off and one past tile and workgroup
+    boundaries, rows that end inside a wavefront's keys, a row of one token.  Against the eager oracle row by
+    row; padded positions exactly zero; and the same bits as the 32-key kernel (reached by also saying
+    "one document per row", which pads nothing more)."""
+    print(f"case B={b} H={h} G={g} S={s} lens={lens}", flush=True)
+    inp = E.make_inputs(2100 + s + b, b, h, g, s, 64, torch.bfloat16)
+    inp = inp[:4] + (TP.mask_dout(inp[4], lens),)
+    got = TP.run_hip(A, *inp, None, 0, lens)
+    o, lse, dq, dk, dv, ds = (t.detach().cpu() for t in got)
+    rds = torch.zeros(h, dtype=torch.float64)
+    for i in range(b):
+        one = [t[i:i + 1] for t in (inp[0], inp[1], inp[2])] + [inp[3], inp[4][i:i + 1]]
+        ro, rlse, rdq, rdk, rdv, rds_i = TP.oracle_eager(*one, None, 0, [lens[i]])
+        TP.compare_all((o[i:i + 1], lse[i:i + 1], dq[i:i + 1], dk[i:i + 1], dv[i:i + 1], rds_i), (ro, rlse, rdq, rdk, rdv, rds_i))
+        rds += rds_i.double()
+        if lens[i] < s:
+            for t in (dq, dk, dv):
+                assert float(t[i, :, lens[i]:].abs().max()) == 0.0
+    TP.check("dsinks", ds, rds.float(), atol=None)
+    if g * b * ((s + 127) // 128) > 512:        # whole key blocks in both kernels: the same order of additions
+        one_document = torch.zeros(b, s, dtype=torch.int32, device=DEV)
+        other = TP.run_hip(A, *inp, None, 0, lens, one_document)
+        for name, x, y in zip(("o", "lse", "dq", "dk", "dv", "dsinks"), got, other):
+            assert torch.equal(x, y), name
+
+
 @pytest.mark.parametrize("b,h,g,s", [
     (1, 16, 2, 2048),      # 32 key blocks: eight slices of four query tiles per 256-key workgroup
     (2, 8, 8, 2304),       # 36 tiles, three slices; the last workgroup of a row holds 256 of its 2304 keys
@@ -257,13 +290,14 @@ def test_dkdv64_route_cut_into_slices_vs_eager_oracle(A, b, h, g, s):
 
 @pytest.mark.parametrize("b,h,g,s", [(1, 64, 8, 16384), (3, 16, 8, 8192 + 64), (16, 8, 4, 1088)])
 def test_dkdv64_route_has_the_bits_of_the_32_key_kernel(A, b, h, g, s):
-    """The same problem with a seqlens array that pads nothing takes attn_bwd_dkdv_kernel (32 keys per
-    wavefront, the general kernel): both add the same products in the same order, so dK and dV agree bit
-    for bit, at GPT-OSS-20B's full 16384-token layer too."""
+    """The same problem with a doc_start array that says "one document per row" takes attn_bwd_dkdv_kernel (32
+    keys per wavefront, the general kernel): both add the same products in the same order, so dK and dV agree
+    bit for bit, at GPT-OSS-20B's full 16384-token layer too."""
     print(f"case B={b} H={h} G={g} S={s}", flush=True)
     q, k, v, sinks, d_out = (t.to(DEV) for t in E.make_inputs(1700 + s, b, h, g, s, 64, torch.bfloat16))
     o, lse = A.attention_forward(q, k, v, sinks, SCALE, None)
-    two = A.attention_backward(q, k, v, sinks, o, lse, d_out, SCALE, None, 0, [s] * b)
+    one_document = torch.zeros(b, s, dtype=torch.int32, device=DEV)
+    two = A.attention_backward(q, k, v, sinks, o, lse, d_out, SCALE, None, 0, None, doc_start=one_document)
     # several runs of the hand-scheduled kernel: its register hazards are handled in the source, not by the
     # compiler, and a violation would show as bits that change from run to run
     for rep in range(4):
