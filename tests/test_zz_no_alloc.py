@@ -95,6 +95,8 @@ def test_static_scratch_backward_matches_workspace_backward(window):
     (1, 17, 1, 200, 128, torch.bfloat16, None),          # 17 query heads per KV head: dQ + dK/dV kernels, static scratch
     (1, 4, 4, 200, 128, torch.bfloat16, None),           # one query head per KV head: the same fallback
     (2, 17, 1, 200, None, torch.bfloat16, [200, 77]),
+    (1, 64, 8, 16384, None, torch.bfloat16, None),       # the headline layer: 64-key dK/dV kernel, 24 of the 48 MiB in use
+    (9, 8, 8, 1024, None, torch.bfloat16, [1024, 1000, 960, 7, 64, 65, 512, 513, 1]),   # the same kernel with padded rows
 ])
 def test_static_scratch_backward_other_routes(b, h, g, s, window, dtype, lens):
     """The routes the two-call test above does not take, each against gptoss_attn_bwd: float32 tensors,
