@@ -306,13 +306,13 @@ def main():
     # What the matrix pipes sustain on this box under the power limit: a loop of nothing but MFMAs (the library's
     # measurement aid), on N(0,1) bf16 operands as the attention kernels see them and on zeros.  Beside it the MFMA
     # work the three kernels execute per second (the dQ kernel recomputes S and dP, the dK/dV kernel adds its
-    # statistics steps: 9 GEMM units + 9.7 % of 4 where 7 are counted).
+    # statistics steps: 9 GEMM units + 6.25 % of 4 where 7 are counted).
     ceiling = mfma_ceiling(stream, sptr)
     ceiling["executed_tflops"] = {
         "fwd": round(2 * unit / (kern["full.fwd"] * 1e-3) / 1e12, 1),
         "dq": round(3 * unit / (kern["full.bwd_dq"] * 1e-3) / 1e12, 1),
-        "dkdv": round(4 * 1.097 * unit / (dkdv_ms * 1e-3) / 1e12, 1),
-        "step": round((9 + 4 * 0.097) * unit / (ms_full * 1e-3) / 1e12, 1)}
+        "dkdv": round(4 * 1.0625 * unit / (dkdv_ms * 1e-3) / 1e12, 1),
+        "step": round((9 + 4 * 0.0625) * unit / (ms_full * 1e-3) / 1e12, 1)}
     out["mfma_ceiling"] = ceiling
 
     if not args.no_cpu_baseline:

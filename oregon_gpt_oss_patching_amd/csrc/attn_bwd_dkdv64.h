@@ -15,7 +15,8 @@
 //
 //   a 64-row query tile against the wavefront's 64 keys = 4 substeps t = (32-row block qb = t / 2,
 //   32-key block nb = t % 2), each
-//     M1(t): S - lse / scale = Q K^T + (statistics step), dP - delta likewise      10 MFMAs, results in VGPRs
+//     M1(t): S - lse / scale = Q K^T + (statistics step), dP - delta likewise      8 MFMAs + 2 for the statistics
+//                                                                                   step of a row block, results in VGPRs
 //     V(t):  P = exp2((S - lse / scale) c), dS = P (dP - delta), -> bf16           16 elements per lane
 //     M2(t): dV^T += dO^T P, dK^T += Q^T dS                                        8 MFMAs, accumulators in AGPRs
 //   issued as a steady stream of slots of 18 MFMAs: slot = { M2(t-1), M1(t+1), V(t), LDS reads }.
@@ -212,17 +213,22 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv64_kernel(const KArgs a) 
     };
     // MFMA j (0..9) of M1(t): S first (its exponentials are what the next slot starts with), each chain led by
     // its statistics step; MFMA j (0..7) of M2(t)
+    // (The statistics step does not depend on the key block: it is issued once per 32-row block, with the first
+    // key block, and both key blocks' chains start from its result.)
+    f32x16 s_init[2], dp_init[2];
     auto m1 = [&](int t, int j) __attribute__((always_inline)) {
         const int qb = t >> 1, nb = t & 1;
         if (j == 0 || j == 5) {
-            f32x16 z;
+            if (nb == 0) {
+                f32x16 z;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) z[i] = 0.0f;
-            if (j == 0) s[t] = mfma_bf16(ast[qb], b_stat_s, z); else dp[t] = mfma_bf16(ast[qb], b_stat_dp, z);
+                for (int i = 0; i < 16; ++i) z[i] = 0.0f;
+                if (j == 0) s_init[qb] = mfma_bf16(ast[qb], b_stat_s, z); else dp_init[qb] = mfma_bf16(ast[qb], b_stat_dp, z);
+            }
         } else if (j < 5) {
-            s[t] = mfma_bf16(aq[qb][j - 1], kf[nb][j - 1], s[t]);
+            s[t] = mfma_bf16(aq[qb][j - 1], kf[nb][j - 1], j == 1 ? s_init[qb] : s[t]);
         } else {
-            dp[t] = mfma_bf16(ag[qb][j - 6], vf[nb][j - 6], dp[t]);
+            dp[t] = mfma_bf16(ag[qb][j - 6], vf[nb][j - 6], j == 6 ? dp_init[qb] : dp[t]);
         }
     };
     // (t = 3 is the substep whose M2 follows a join of control flow: the top of the loop body and the drain;
