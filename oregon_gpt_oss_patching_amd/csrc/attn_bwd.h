@@ -663,8 +663,9 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_bwd_dq_kernel(co
     const int t_lo = max(key_lo, ds_b0) / kTile;
     const int t_hi = hi > 0 ? (hi + kTile - 1) / kTile : 0;
 
-    const int wpos0 = q_offset + qw0;
-    const int wpos1 = min(q_offset + min(a.Sq, qw0 + WM) - 1, q_len - 1);
+    // (wave-uniform values, said so to the compiler: the tile classification then branches on scalar conditions)
+    const int wpos0 = __builtin_amdgcn_readfirstlane(q_offset + qw0);
+    const int wpos1 = __builtin_amdgcn_readfirstlane(min(q_offset + min(a.Sq, qw0 + WM) - 1, q_len - 1));
 
     const bf16 *kbase = a.k + (int64_t)b * a.ks.b + (int64_t)g * a.ks.h;
     const bf16 *vbase = a.v + (int64_t)b * a.vs.b + (int64_t)g * a.vs.h;
