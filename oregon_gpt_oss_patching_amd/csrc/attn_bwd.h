@@ -752,8 +752,8 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_bwd_dq_kernel(co
     auto issue = [&](int it) {
         const int stage = it % NS;
         if (next_row0 + kTile <= a.Skv) {
-            tile_async_inner(smem[stage][0], ktile, klane, w);
-            tile_async_inner(smem[stage][1], vtile, vlane, w);
+            tile_async_inner(smem[stage][0], ktile, klane, w_s);      // (scalar wave index: the LDS base is formed on the scalar unit)
+            tile_async_inner(smem[stage][1], vtile, vlane, w_s);
         } else {
             const int fl = fresh_lane();
             tile_async(smem[stage][0], kbase, a.ks.s, next_row0, a.Skv, fl, w_s);

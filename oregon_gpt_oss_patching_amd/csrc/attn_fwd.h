@@ -268,13 +268,14 @@ __global__ __launch_bounds__(256, (NQB == 1 ? 3 : 2)) void attn_fwd_kernel(const
     // K / V tiles are requested in order; the pointers to the next tile's first row advance by
     // one tile per request.  Only a tile that sticks out of the tensor takes the clamping copy.
     const AsyncLaneOffsets klane = make_async_offsets(a.ks.s, lane, w), vlane = make_async_offsets(a.vs.s, lane, w);
+    const int w_s = __builtin_amdgcn_readfirstlane(w);
     const bf16 *ktile = kbase, *vtile = vbase;
     int next_row0 = 0;
     auto issue = [&](int it) __attribute__((always_inline)) {
         const int stage = it % NS;
         if (next_row0 + kTile <= a.Skv) {
-            tile_async_inner(smem[stage][0], ktile, klane, w);
-            tile_async_inner(smem[stage][1], vtile, vlane, w);
+            tile_async_inner(smem[stage][0], ktile, klane, w_s);      // (scalar wave index: the LDS base is formed on the scalar unit)
+            tile_async_inner(smem[stage][1], vtile, vlane, w_s);
         } else {
             tile_async(smem[stage][0], kbase, a.ks.s, next_row0, a.Skv, lane, w);
             tile_async(smem[stage][1], vbase, a.vs.s, next_row0, a.Skv, lane, w);
