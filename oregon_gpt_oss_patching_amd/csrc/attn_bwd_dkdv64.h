@@ -147,29 +147,42 @@ __global__ __launch_bounds__(256, 1) void attn_bwd_dkdv64_kernel(const KArgs a) 
     const uint32_t stat_voff = w * (C::kWaveRows * 16) + lane * 4;
     const uint32_t stat_dst = __builtin_amdgcn_readfirstlane(C::kStatOff - w * (C::kWaveRows * kRowBytes) + w * (C::kWaveRows * 16));
     int iss_h = 0, iss_left = n_it;
-    const int i0_first = max(qt_hi - 1, 0) * kTile;      // (an empty slice requests nothing: n_it is 0)
-    const bf16 *qtile = a.q + (int64_t)b * a.qs.b + (int64_t)(g * a.r) * a.qs.h + (int64_t)i0_first * a.qs.s;
-    const bf16 *gtile = a.d_o + (int64_t)b * a.dos.b + (int64_t)(g * a.r) * a.dos.h + (int64_t)i0_first * a.dos.s;
-    const u32x4 *stat_src = a.split + ((int64_t)b * a.H + (int64_t)g * a.r) * a.Sq + i0_first;     // wave-uniform
-    const int64_t q_step = a.qs.h, q_wrap = a.qs.h - (int64_t)a.r * a.qs.h - (int64_t)kTile * a.qs.s;
-    const int64_t g_step = a.dos.h, g_wrap = a.dos.h - (int64_t)a.r * a.dos.h - (int64_t)kTile * a.dos.s;
-    const int64_t s_step = a.Sq, s_wrap = (int64_t)a.Sq - (int64_t)a.r * a.Sq - kTile;
+    // The walk moves 32-bit byte offsets (the lanes' own, one vector add each per tile) over fixed bases: the
+    // lowest tile of the slice, first head of the group.  Scalar instructions are the expensive ones for a
+    // wavefront that has its SIMD to itself (about 8 cycles of issue each, a vector add 4), and 64-bit pointer
+    // walks take many.  The host takes this kernel only when every such offset fits (dkdv64_route).
+    const int n_tiles = a.Sq / kTile;
+    const int t_base = max(0, min(qt_hi - nq, n_tiles - 1));          // (an empty slice requests tile t_base over and over)
+    const int t_first = max(0, nq - 1);                                // tiles above t_base where the walk starts
+    const bf16 *qbase = a.q + (int64_t)b * a.qs.b + (int64_t)(g * a.r) * a.qs.h + (int64_t)(t_base * kTile) * a.qs.s;
+    const bf16 *gbase = a.d_o + (int64_t)b * a.dos.b + (int64_t)(g * a.r) * a.dos.h + (int64_t)(t_base * kTile) * a.dos.s;
+    const u32x4 *stat_base = a.split + ((int64_t)b * a.H + (int64_t)g * a.r) * a.Sq + t_base * kTile;     // wave-uniform
+    uint32_t qoff0 = qlane.off[0] + (uint32_t)(t_first * kTile) * (uint32_t)a.qs.s * 2u, qoff1 = qlane.off[1] + (uint32_t)(t_first * kTile) * (uint32_t)a.qs.s * 2u;
+    uint32_t goff0 = glane.off[0] + (uint32_t)(t_first * kTile) * (uint32_t)a.dos.s * 2u, goff1 = glane.off[1] + (uint32_t)(t_first * kTile) * (uint32_t)a.dos.s * 2u;
+    uint32_t soff = stat_voff + (uint32_t)(t_first * kTile) * 16u;
+    // per request: on to the next head, or (after the last head of the group) back to the first head of the tile below
+    const uint32_t q_step = (uint32_t)a.qs.h * 2u, q_wrap = 0u - ((uint32_t)(a.r - 1) * (uint32_t)a.qs.h + (uint32_t)kTile * (uint32_t)a.qs.s) * 2u;
+    const uint32_t g_step = (uint32_t)a.dos.h * 2u, g_wrap = 0u - ((uint32_t)(a.r - 1) * (uint32_t)a.dos.h + (uint32_t)kTile * (uint32_t)a.dos.s) * 2u;
+    const uint32_t s_step = (uint32_t)a.Sq * 16u, s_wrap = 0u - ((uint32_t)(a.r - 1) * (uint32_t)a.Sq + (uint32_t)kTile) * 16u;
     // copy `which` (0..4) of the current request into the stage at `dst`; advance() moves on to the next tile
     auto issue_one = [&](uint32_t dst, int which) __attribute__((always_inline)) {
-        if (which == 0) lds_dma16_plus<0>(dst, qtile, qlane.off[0]);
-        if (which == 1) lds_dma16_plus<8 * kRowBytes>(dst, qtile, qlane.off[1]);
-        if (which == 2) lds_dma16_plus<kStageTileBytes>(dst, gtile, glane.off[0]);
-        if (which == 3) lds_dma16_plus<kStageTileBytes + 8 * kRowBytes>(dst, gtile, glane.off[1]);
-        if (which == 4) lds_dma4(dst + stat_dst, stat_src, stat_voff);
+        if (which == 0) lds_dma16_plus<0>(dst, qbase, qoff0);
+        if (which == 1) lds_dma16_plus<8 * kRowBytes>(dst, qbase, qoff1);
+        if (which == 2) lds_dma16_plus<kStageTileBytes>(dst, gbase, goff0);
+        if (which == 3) lds_dma16_plus<kStageTileBytes + 8 * kRowBytes>(dst, gbase, goff1);
+        if (which == 4) lds_dma4_at(dst, stat_dst, stat_base, soff);
     };
     auto advance = [&]() __attribute__((always_inline)) {
         const bool more = iss_left > 1;                 // another tile to request after this one
         const bool wrap = iss_h + 1 == a.r;
-        qtile += more ? (wrap ? q_wrap : q_step) : 0;
-        gtile += more ? (wrap ? g_wrap : g_step) : 0;
-        stat_src += more ? (wrap ? s_wrap : s_step) : 0;
+        const uint32_t dq_ = more ? (wrap ? q_wrap : q_step) : 0u;
+        const uint32_t dg_ = more ? (wrap ? g_wrap : g_step) : 0u;
+        const uint32_t ds_ = more ? (wrap ? s_wrap : s_step) : 0u;
+        qoff0 += dq_; qoff1 += dq_;
+        goff0 += dg_; goff1 += dg_;
+        soff += ds_;
         iss_h = wrap ? 0 : iss_h + 1;
-        iss_left = max(iss_left - 1, 0);
+        iss_left -= 1;
     };
     auto issue = [&](uint32_t dst) __attribute__((always_inline)) {
 #pragma unroll

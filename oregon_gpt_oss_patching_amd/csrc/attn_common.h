@@ -207,6 +207,10 @@ __device__ __forceinline__ void lds_dma16_plus(uint32_t lds_base, const void *gb
 __device__ __forceinline__ void lds_dma4(uint32_t lds_base, const void *gbase, uint32_t voff) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(lds_base), "v"(voff), "s"(gbase) : "memory");
 }
+// the same with the LDS base given as the sum of two scalar registers, formed in M0 by one instruction
+__device__ __forceinline__ void lds_dma4_at(uint32_t lds_base, uint32_t lds_off, const void *gbase, uint32_t voff) {
+    asm volatile("s_add_u32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %2, %3" ::"s"(lds_base), "s"(lds_off), "v"(voff), "s"(gbase) : "memory", "scc");
+}
 
 // Issues the 4-wavefront asynchronous copy of tile rows [row0, row0+64) (rows at or
 // beyond row_end re-read the last valid row: their products are masked, they only

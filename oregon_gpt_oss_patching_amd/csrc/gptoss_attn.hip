@@ -117,8 +117,18 @@ int dkdv_parts_for(const gptoss_attn_params *p) {
 // whole: at least 257 workgroups of 256 keys, and the same bits as the 32-key kernel), or rows of 2048 keys
 // or more that the host cuts into `parts` slices anyway (the same number of slices as the 32-key kernel
 // would get, so the scratch is the same; -15 % at S = 2048 ... 8192).
+// (The kernel walks Q, dO and the row statistics of one KV head's group of query heads with 32-bit byte
+// offsets from the group's first row: head strides must not be negative and the group's span must stay
+// below 2^31 bytes; anything else takes the 32-key kernel.)
+bool walk_fits_32_bits(const gptoss_attn_strides &s, int64_t heads, int64_t rows) {
+    return s.h >= 0 && ((heads - 1) * s.h + rows * s.s) * 2 < ((int64_t)1 << 31);
+}
 bool dkdv64_route(const gptoss_attn_params *p, int parts) {
     const int64_t blocks = (int64_t)p->G * p->B * ((p->Skv + kDkdvKeys - 1) / kDkdvKeys);
+    const int64_t heads = p->H / p->G;
+    if (!walk_fits_32_bits(p->q_stride, heads, p->Sq) || !walk_fits_32_bits(p->do_stride, heads, p->Sq) ||
+        heads * p->Sq * 16 >= ((int64_t)1 << 31))
+        return false;
     return p->dtype == GPTOSS_ATTN_BF16 && effective_window(p) == 0 && !p->doc_start && p->q_offset == 0 &&
            !p->q_offset_dev && p->Sq == p->Skv && p->Sq % kTile == 0 && (blocks > 512 || (parts > 1 && p->Skv >= 2048));
 }

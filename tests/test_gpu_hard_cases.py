@@ -306,3 +306,29 @@ def test_dkdv64_route_has_the_bits_of_the_32_key_kernel(A, b, h, g, s):
         for name, x, y in zip(("dq", "dk", "dv", "dsinks"), one, two):
             assert torch.isfinite(x.float()).all(), (name, rep)
             assert torch.equal(x, y), (name, rep)
+
+
+def test_rows_too_far_apart_for_the_64_key_kernel_take_the_general_one(A):
+    """The 64-key dK/dV kernel walks Q and dO with 32-bit byte offsets from the first row of a KV head's group; a
+    view whose rows lie 512 KB apart spans 2 GiB at 4096 rows, so the host gives that problem to the general
+    kernel.  Both add the same products in the same order: the results are those of the packed tensors, bit
+    for bit."""
+    b, h, g, s = 1, 64, 8, 4096
+    print(f"case B={b} H={h} G={g} S={s} with a sequence stride of 262144 elements", flush=True)
+    q, k, v, sinks, d_out = (t.to(DEV) for t in E.make_inputs(1811, b, h, g, s, 64, torch.bfloat16))
+    o, lse = A.attention_forward(q, k, v, sinks, SCALE, None)
+    want = A.attention_backward(q, k, v, sinks, o, lse, d_out, SCALE, None)
+
+    def far_apart(t, seq_dim):
+        big = torch.zeros(s, 262144, dtype=t.dtype, device=DEV)           # 2 GiB
+        view = big[:, :h * 64].view(b, s, h, 64)                          # [B, S, H, D]
+        if seq_dim == 2:
+            view = view.permute(0, 2, 1, 3)                               # [B, H, S, D]
+        view.copy_(t)
+        assert view.shape == t.shape and view.stride(seq_dim) == 262144
+        return view
+
+    got = A.attention_backward(far_apart(q, 2), k, v, sinks, o, lse, far_apart(d_out, 1), SCALE, None)
+    torch.cuda.synchronize()
+    for name, x, y in zip(("dq", "dk", "dv", "dsinks"), got, want):
+        assert torch.equal(x, y), name
