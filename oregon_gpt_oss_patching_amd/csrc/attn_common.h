@@ -182,7 +182,8 @@ __device__ __forceinline__ int swz(int r) { return (((r >> 1) & 1) << 2) | (((r 
 typedef __attribute__((address_space(3))) void lds_void_t;
 typedef __attribute__((address_space(1))) const void glb_void_t;
 
-// The copy instruction written as inline assembly (used by attn_bwd_dkdv64_kernel only).  Issued through
+// The copy instruction written as inline assembly (used by the hand-pipelined kernels, attn_bwd_dkdv64_kernel
+// and attn_fwd_pipe_kernel).  Issued through
 // the compiler's builtin, every LDS read that follows a copy is made to wait for ALL outstanding copies (the
 // compiler cannot tell which LDS bytes a copy writes, and a workgroup barrier waits for them as well), which
 // turns a three-stage pipeline into "issue, wait for what was just issued, compute".  Hidden in the
@@ -190,8 +191,10 @@ typedef __attribute__((address_space(1))) const void glb_void_t;
 // business: wait_vmcnt<N>() before the barrier that hands a stage to its readers, and a barrier
 // between the last read of a stage and the copy that overwrites it.  (Compiler-generated vmcnt waits
 // for its own loads stay correct: loads return in order, so unknown extra loads only make such a wait
-// longer.)  M0 holds the wave-uniform LDS base; nothing else in these kernels uses M0.  The kernels with
-// two wavefronts per SIMD keep the builtin: there the hidden form measured slower.
+// longer.)  M0 holds the wave-uniform LDS base; nothing else in these kernels uses M0.  The kernels whose key
+// loops are scheduled by the compiler (attn_fwd_kernel, attn_bwd_dq_kernel) keep the builtin: their wavefronts
+// alternate between stretches of MFMAs and stretches of vector work whatever the copies do, and the hidden
+// form measured the same or slower there.
 // lane L's 16 bytes at gbase + voff land at lds_base + 16 * L
 __device__ __forceinline__ void lds_dma16(uint32_t lds_base, const void *gbase, uint32_t voff) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_base), "v"(voff), "s"(gbase) : "memory");

@@ -332,3 +332,27 @@ def test_rows_too_far_apart_for_the_64_key_kernel_take_the_general_one(A):
     torch.cuda.synchronize()
     for name, x, y in zip(("dq", "dk", "dv", "dsinks"), got, want):
         assert torch.equal(x, y), name
+
+
+@pytest.mark.parametrize("b,h,g,s", [(2, 8, 2, 64), (2, 16, 4, 128), (1, 32, 8, 192), (3, 16, 4, 1088), (1, 64, 8, 16384)])
+def test_pipelined_forward_vs_the_general_forward_kernel(A, b, h, g, s):
+    """Plain full-causal problems take attn_fwd_pipe_kernel (hand-scheduled key loop, the row's softmax reference
+    from a pass of its own over the first tile); the same problem with a doc_start array that says "one document
+    per row" takes attn_fwd_kernel.  Both follow the same formulas with the row sums taken in a different order,
+    so lse agrees to a few units of its last fp32 place and O to one bf16 rounding; rows of 1, 2 and 3 key
+    tiles take the kernel's short paths (no loop, no steady state).  The hand-scheduled kernel gives the same
+    bits on every run."""
+    print(f"case B={b} H={h} G={g} S={s}", flush=True)
+    q, k, v, sinks, _ = (t.to(DEV) for t in E.make_inputs(1900 + s, b, h, g, s, 64, torch.bfloat16))
+    one_document = torch.zeros(b, s, dtype=torch.int32, device=DEV)
+    o_ref, lse_ref = A.attention_forward(q, k, v, sinks, SCALE, None, doc_start=one_document)
+    o, lse = A.attention_forward(q, k, v, sinks, SCALE, None)
+    torch.cuda.synchronize()
+    assert torch.isfinite(o.float()).all() and torch.isfinite(lse).all()
+    assert (lse - lse_ref).abs().max().item() <= 1e-5
+    err = (o.float() - o_ref.float()).abs()
+    assert (err <= 2.0 ** -7 * o_ref.float().abs() + 1e-6).all(), err.max().item()      # one bf16 unit in the last place
+    for rep in range(3):
+        o2, lse2 = A.attention_forward(q, k, v, sinks, SCALE, None)
+        torch.cuda.synchronize()
+        assert torch.equal(o, o2) and torch.equal(lse, lse2), rep
