@@ -1,7 +1,8 @@
 // Forward kernel for the plain full-causal case (bf16, no window, no packed or padded rows, no query
-// offset, Sq == Skv a multiple of 64, query heads per KV head a multiple of 4): the same arithmetic in the
-// same order as attn_fwd_kernel<4, 2> (attn_fwd.h; the reference's `_attn_fwd`, attention_kernel.py:11-100),
-// so the same bits, with the interior key tiles software-pipelined by hand.
+// offset, Sq == Skv a multiple of 64, query heads per KV head a multiple of 4): the formulas of
+// attn_fwd_kernel<4, 2> (attn_fwd.h; the reference's `_attn_fwd`, attention_kernel.py:11-100) with the
+// interior key tiles software-pipelined by hand.  Against that kernel only the order of the row sums of a
+// row's first tile differs: lse agrees to a few units of its last place, O to one bf16 rounding.
 //
 // Why.  Two wavefronts share a SIMD.  attn_fwd_kernel's wavefront issues its MFMAs in clumps of eight with a
 // softmax step (about 120 vector instructions, no MFMA) between them; while one wavefront sits in such a
@@ -19,8 +20,10 @@
 // right after their last use, one slot before their first.  The next tile must have landed before the
 // third slot of a tile (which loads its first K fragments), so the iteration's barrier sits there; with four
 // LDS stages the copy requested at that barrier is two tiles ahead, as in attn_fwd_kernel.
-// The first tile of a row (it sets the softmax reference, see fwd_tile_lean) and the diagonal tile (masked)
-// go through attn_fwd.h's tile functions.
+// The softmax reference of a row (see fwd_tile_lean) is the sink logit or the largest logit of the row's first
+// tile, taken by a pass over that tile that forms the logits and nothing else; the tile then goes through the
+// loop like the others.  The diagonal tile (masked) goes through attn_fwd.h's fwd_tile_lean, and so does the
+// rare second pass of a workgroup whose frozen reference turned out too low (fwd_tile on every tile).
 #pragma once
 #include <type_traits>
 
