@@ -1,5 +1,5 @@
-// Forward kernel for the plain full-causal case (bf16, no window, no packed or padded rows, no query
-// offset, Sq == Skv a multiple of 64, query heads per KV head a multiple of 4): the formulas of
+// Forward kernel for the plain full-causal case (bf16, no window, no packed rows, no query offset, right-padded
+// batch rows allowed, Sq == Skv a multiple of 64, query heads per KV head a multiple of 4): the formulas of
 // attn_fwd_kernel<4, 2> (attn_fwd.h; the reference's `_attn_fwd`, attention_kernel.py:11-100) with the
 // interior key tiles software-pipelined by hand.  Against that kernel only the order of the row sums of a
 // row's first tile differs: lse agrees to a few units of its last place, O to one bf16 rounding.
@@ -22,8 +22,9 @@
 // LDS stages the copy requested at that barrier is two tiles ahead, as in attn_fwd_kernel.
 // The softmax reference of a row (see fwd_tile_lean) is the sink logit or the largest logit of the row's first
 // tile, taken by a pass over that tile that forms the logits and nothing else; the tile then goes through the
-// loop like the others.  The diagonal tile (masked) goes through attn_fwd.h's fwd_tile_lean, and so does the
-// rare second pass of a workgroup whose frozen reference turned out too low (fwd_tile on every tile).
+// loop like the others.  The diagonal tile (masked) goes through attn_fwd.h's fwd_tile_lean; rows of a single
+// key tile, and the rare second pass of a workgroup whose frozen reference turned out too low, go through one
+// loop of exact steps (fwd_tile).
 #pragma once
 #include <type_traits>
 
@@ -36,6 +37,12 @@ struct FwdPipe {
     static constexpr int kStageBytes = 2 * kStageTileBytes;       // K tile, V tile
 };
 
+// PADDED: right-padded batch rows (seqlens): a row of the batch is a shorter row.  Workgroups past its end write
+// O = 0 and lse = sink and do nothing else; in the workgroup that holds its end the rows past it run along
+// unmasked through the interior tiles (their logits are garbage but finite or at worst NaN, and stay in their own
+// lanes) and are set to that same result before the epilogue; keys past the end exist only in the diagonal
+// tile, whose tile function masks them.
+template <bool PADDED>
 __global__ __launch_bounds__(256, 2) void attn_fwd_pipe_kernel(const KArgs a) {
     constexpr int NS = FwdPipe::NS;
     constexpr int SB = FwdPipe::kStageBytes;
@@ -58,21 +65,19 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_pipe_kernel(const KArgs a) {
     const int head = g * a.r + hc * 4 + w;
     const int qw0 = qt * kTile;                    // the four wavefronts hold the same 64 rows of four heads
     const int n_it = qt + 1;                       // key tiles 0 .. qt, the last one on the diagonal
+    const int len = PADDED ? max(0, min(a.Sq, a.seqlens[b])) : a.Sq;      // rows and keys from len on do not exist
+    const bool wg_dead = PADDED && qw0 >= len;
 
     const bf16 *kbase = a.k + (int64_t)b * a.ks.b + (int64_t)g * a.ks.h;
     const bf16 *vbase = a.v + (int64_t)b * a.vs.b + (int64_t)g * a.vs.h;
 
     bf16x8 qf[2][4];
-    int pq[2];
-    unsigned wl[2];
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) {
         const int row = qw0 + 32 * qb + l32;
         const bf16 *qrow = a.q + (int64_t)b * a.qs.b + (int64_t)head * a.qs.h + (int64_t)row * a.qs.s;
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks) qf[qb][ks] = as_bf16x8(*reinterpret_cast<const u32x4 *>(qrow + 16 * ks + 8 * half));
-        pq[qb] = row;
-        wl[qb] = 0x3fffffffu;
     }
 
     const float c = a.scale_log2;
@@ -126,19 +131,20 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_pipe_kernel(const KArgs a) {
         __syncthreads();
         issue();
     };
-    const int wrel_diag = qw0 - qt * kTile;        // 0: the diagonal tile starts at the wavefront's first row
-    auto masked_args = [&](int n0, int (&dbase)[2]) __attribute__((always_inline)) {
+    // Rows of a single key tile (the diagonal one) have no interior tile: they go straight to the exact pass below.
+    const bool pipelined = !wg_dead && n_it >= 2;
+    if (!pipelined) {
+        // (also the state a workgroup without rows ends with: nothing requested, nothing attended)
 #pragma unroll
-        for (int qb = 0; qb < 2; ++qb) dbase[qb] = pq[qb] - n0;
-    };
-
-    reset();
-    arrive();
-    if (n_it == 1) {
-        int dbase[2];
-        masked_args(0, dbase);
-        fwd_tile<true, 2>(smem_base, smem_base + kStageTileBytes, lo, qf, o, m, l, c, lane, dbase, wl, 0x3fffffffu, a.Skv, wrel_diag);
+        for (int qb = 0; qb < 2; ++qb) {
+            m[qb] = sink2;
+            l[qb] = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) { o[qb][0][i] = 0.0f; o[qb][1][i] = 0.0f; }
+        }
     } else {
+        reset();
+        arrive();
         // The softmax reference of a row: the sink logit or the largest logit of the row's first tile
         // (ref :53, :79-81 after one tile), from a pass over that tile that forms the logits and nothing else
         // (16 MFMAs per row block, against 32 for each of its tiles).  The tile then goes through the pipelined
@@ -167,7 +173,7 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_pipe_kernel(const KArgs a) {
     }
     float nm[2] = {-m[0], -m[1]};
 
-    if (n_it >= 2) {
+    if (pipelined) {
 #define GPTOSS_FP_FENCE() __builtin_amdgcn_sched_barrier(0)
         // (an MFMA's result is not needed before the next slot, and instruction selection would place it there,
         // across the fences, which only bind the scheduler that runs afterwards: an empty volatile statement
@@ -287,39 +293,60 @@ __global__ __launch_bounds__(256, 2) void attn_fwd_pipe_kernel(const KArgs a) {
     int pq_b[2];
     unsigned wl_b[2];
 #pragma unroll
-    for (int qb = 0; qb < 2; ++qb) { pq_b[qb] = qw0 + 32 * qb + l32_b; wl_b[qb] = 0x3fffffffu; }
+    for (int qb = 0; qb < 2; ++qb) { pq_b[qb] = qw0 + 32 * qb + l32_b < len ? qw0 + 32 * qb + l32_b : -0x40000000; wl_b[qb] = 0x3fffffffu; }   // (hugely negative: nothing is visible to a row that does not exist)
     auto masked_args_b = [&](int n0, int (&dbase)[2]) __attribute__((always_inline)) {
 #pragma unroll
         for (int qb = 0; qb < 2; ++qb) dbase[qb] = pq_b[qb] - n0;
     };
-    if (n_it >= 2) {
+    if (pipelined) {
         const int n0 = qt * kTile;
         const uint32_t ksm = smem_base + (qt & (NS - 1)) * SB;
         int dbase[2];
         masked_args_b(n0, dbase);
-        fwd_tile_lean<true, 2>(ksm, ksm + kStageTileBytes, lo_b, qf, o, nm, l, c, lane_b, dbase, wl_b, 0x3fffffffu, a.Skv - n0, wrel_diag);
+        fwd_tile_lean<true, 2>(ksm, ksm + kStageTileBytes, lo_b, qf, o, nm, l, c, lane_b, dbase, wl_b, 0x3fffffffu, len - n0, 0);
     }
 
     // A sum beyond 2^96 (or not finite): some logit stood 95 or more above its row's frozen reference; the
     // workgroup repeats its key loop with the exact online-softmax step on every tile (see attn_fwd_kernel).
+    // rows that do not exist: nothing attended, whatever the interior tiles made of them
+    auto clear_dead_rows = [&]() __attribute__((always_inline)) {
+        if constexpr (PADDED) {
+#pragma unroll
+            for (int qb = 0; qb < 2; ++qb) {
+                const bool dead_row = pq_b[qb] < 0;
+                m[qb] = dead_row ? sink2 : m[qb];
+                l[qb] = dead_row ? 0.0f : l[qb];
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    o[qb][0][i] = dead_row ? 0.0f : o[qb][0][i];
+                    o[qb][1][i] = dead_row ? 0.0f : o[qb][1][i];
+                }
+            }
+        }
+    };
+    clear_dead_rows();
+    // A sum beyond 2^96 (or not finite): some logit stood 95 or more above its row's frozen reference; the
+    // workgroup repeats its key loop with the exact online-softmax step on every tile (see attn_fwd_kernel; the
+    // masked form of the step for every tile: this pass is rare and the kernel stays small).  Rows of a single
+    // tile take this pass as their only one.
     bool unsafe = false;
 #pragma unroll
     for (int qb = 0; qb < 2; ++qb) unsafe = unsafe || !(l[qb] < 0x1p96f);
-    if (__syncthreads_or(unsafe)) {
-        wait_vmcnt<0>();          // the repeated copies of the last requests
-        __syncthreads();
+    const bool second_pass = pipelined && __syncthreads_or(unsafe);
+    if (second_pass || (!pipelined && !wg_dead)) {
+        if (second_pass) {
+            wait_vmcnt<0>();      // the repeated copies of the last requests
+            __syncthreads();
+        }
         reset();
         for (int it = 0; it < n_it; ++it) {
             arrive();
             const uint32_t ksm = smem_base + (it & (NS - 1)) * SB;
-            if (it < qt) {
-                fwd_tile<false, 2>(ksm, ksm + kStageTileBytes, lo_b, qf, o, m, l, c, lane_b, pq_b, wl_b, 0u, 0, 0);
-            } else {
-                int dbase[2];
-                masked_args_b(it * kTile, dbase);
-                fwd_tile<true, 2>(ksm, ksm + kStageTileBytes, lo_b, qf, o, m, l, c, lane_b, dbase, wl_b, 0x3fffffffu, a.Skv - it * kTile, wrel_diag);
-            }
+            int dbase[2];
+            masked_args_b(it * kTile, dbase);
+            fwd_tile<true, 2>(ksm, ksm + kStageTileBytes, lo_b, qf, o, m, l, c, lane_b, dbase, wl_b, 0x3fffffffu, len - it * kTile, qw0 - it * kTile);
         }
+        clear_dead_rows();
     }
 
     // epilogue: z = l + exp(sink - m); O = acc / z; M = m + log z   (ref :93-98)

@@ -134,10 +134,10 @@ bool dkdv64_route(const gptoss_attn_params *p, int parts) {
            !p->q_offset_dev && p->Sq == p->Skv && p->Sq % kTile == 0 && (blocks > 512 || (parts > 1 && p->Skv >= 2048));
 }
 
-// The hand-pipelined forward kernel (attn_fwd_pipe.h) takes the plain full-causal case: every row of every
-// workgroup exists, every key tile but the last of a row is interior, all four wavefronts have a head.
+// The hand-pipelined forward kernel (attn_fwd_pipe.h) takes the plain full-causal case (right-padded batch rows
+// included): every key tile but the last of a row is interior, all four wavefronts have a head.
 bool fwd_pipe_route(const gptoss_attn_params *p) {
-    return p->dtype == GPTOSS_ATTN_BF16 && effective_window(p) == 0 && !p->doc_start && !p->seqlens && p->q_offset == 0 &&
+    return p->dtype == GPTOSS_ATTN_BF16 && effective_window(p) == 0 && !p->doc_start && p->q_offset == 0 &&
            !p->q_offset_dev && p->Sq == p->Skv && p->Sq % kTile == 0 && (p->H / p->G) % 4 == 0;
 }
 
@@ -338,7 +338,7 @@ int gptoss_attn_fwd(const gptoss_attn_params *p, void *stream) {
         return launch(attn_f32_fwd_kernel, f32_grid((int64_t)a.B * a.H * ((a.Sq + 31) / 32)), 256, st, a);
     const int hpb = hpb_for(a.r), qb = query_blocks_for(a.window);
     const int64_t grid = q_outer_grid(a, hpb, qb);
-    if (fwd_pipe_route(p)) return launch(attn_fwd_pipe_kernel, grid, 256, st, a);
+    if (fwd_pipe_route(p)) return a.seqlens ? launch(attn_fwd_pipe_kernel<true>, grid, 256, st, a) : launch(attn_fwd_pipe_kernel<false>, grid, 256, st, a);
 #define GPTOSS_LAUNCH_FWD(HPB, QB) launch(attn_fwd_kernel<HPB, QB>, grid, 256, st, a)
     if (qb == 2) return hpb == 4 ? GPTOSS_LAUNCH_FWD(4, 2) : hpb == 2 ? GPTOSS_LAUNCH_FWD(2, 2) : GPTOSS_LAUNCH_FWD(1, 2);
     return hpb == 4 ? GPTOSS_LAUNCH_FWD(4, 1) : hpb == 2 ? GPTOSS_LAUNCH_FWD(2, 1) : GPTOSS_LAUNCH_FWD(1, 1);

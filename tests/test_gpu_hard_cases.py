@@ -356,3 +356,28 @@ def test_pipelined_forward_vs_the_general_forward_kernel(A, b, h, g, s):
         o2, lse2 = A.attention_forward(q, k, v, sinks, SCALE, None)
         torch.cuda.synchronize()
         assert torch.equal(o, o2) and torch.equal(lse, lse2), rep
+
+
+@pytest.mark.parametrize("b,h,g,s,lens", [
+    (5, 16, 4, 1088, [1088, 1, 577, 1024, 64]),        # a whole row, one token, an end inside a tile, on a tile boundary, one tile
+    (3, 32, 8, 256, [65, 192, 0]),                     # ends in the second tile of a row; a row with nothing in it
+])
+def test_pipelined_forward_right_padded_rows(A, b, h, g, s, lens):
+    """Right-padded batch rows through attn_fwd_pipe_kernel<true>: the workgroup that holds a row's end lets the rows
+    past it run unmasked through the interior tiles and clears them afterwards, workgroups past the end only write
+    their result.  Against the general kernel (doc_start of zeros): rows that exist agree as in the unpadded case,
+    rows that do not are exactly O = 0, with lse the sink logit."""
+    print(f"case B={b} H={h} G={g} S={s} lens={lens}", flush=True)
+    q, k, v, sinks, _ = (t.to(DEV) for t in E.make_inputs(2100 + s, b, h, g, s, 64, torch.bfloat16))
+    one_document = torch.zeros(b, s, dtype=torch.int32, device=DEV)
+    o_ref, lse_ref = A.attention_forward(q, k, v, sinks, SCALE, None, 0, lens, doc_start=one_document)
+    o, lse = A.attention_forward(q, k, v, sinks, SCALE, None, 0, lens)
+    torch.cuda.synchronize()
+    assert torch.isfinite(o.float()).all() and torch.isfinite(lse).all()
+    assert (lse - lse_ref).abs().max().item() <= 1e-5
+    err = (o.float() - o_ref.float()).abs()
+    assert (err <= 2.0 ** -7 * o_ref.float().abs() + 1e-6).all(), err.max().item()
+    for i, n in enumerate(lens):
+        assert (o[i, n:] == 0).all()
+        assert torch.equal(lse[i, :, n:], lse_ref[i, :, n:])                         # the sink logit (through log2 and back)
+        assert (lse[i, :, n:] - sinks.float().view(h, 1)).abs().max().item() <= 1e-6 if n < s else True

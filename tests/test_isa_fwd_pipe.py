@@ -16,7 +16,7 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 CSRC = os.path.join(ROOT, "oregon_gpt_oss_patching_amd", "csrc")
-KERNEL = "attn_fwd_pipe_kernel"
+KERNEL = "attn_fwd_pipe_kernel"        # both instantiations are checked (with and without padded batch rows)
 
 
 def _hipcc():
@@ -26,15 +26,16 @@ def _hipcc():
     return None
 
 
-@pytest.fixture(scope="module")
-def kernel_lines(tmp_path_factory):
+@pytest.fixture(scope="module", params=[False, True], ids=["plain", "padded_rows"])
+def kernel_lines(tmp_path_factory, request):
     hipcc = _hipcc()
     if hipcc is None:
         pytest.skip("hipcc not found")
     from oregon_gpt_oss_patching_amd import build as B
     d = tmp_path_factory.mktemp("isa_fwd")
     src = d / "unit.hip"
-    src.write_text('#include "%s"\n' % os.path.join(CSRC, "attn_fwd_pipe.h"))
+    src.write_text('#include "%s"\ntemplate __global__ void gptoss::attn_fwd_pipe_kernel<%s>(const gptoss::KArgs);\n'
+                   % (os.path.join(CSRC, "attn_fwd_pipe.h"), "true" if request.param else "false"))
     out = d / "unit.s"
     flags = [f for f in B.HIPCC_FLAGS if f not in ("-fPIC", "-shared")]
     proc = subprocess.run([hipcc, *flags, "-S", "--cuda-device-only", "-o", str(out), str(src)], capture_output=True, text=True)
