@@ -145,11 +145,16 @@ def main():
     ap.add_argument("--summarize", nargs="+", metavar="DIR",
                     help="rocprofv3 output directories (each holding one *_results.db) of runs made with --layers L "
                          "--copy-calibration; writes the summary given by --out-md and updates the traffic record")
+    ap.add_argument("--stream-probe", action="store_true",
+                    help="instead of the benchmark: time the synthetic instruction streams of gptoss_attn_stream_probe and print, "
+                         "as markdown, the matrix-pipe cycles per MFMA each instruction mix needs at 1, 2 and 3 wavefronts per SIMD")
     ap.add_argument("--summary-layer", choices=("full", "window"))
     ap.add_argument("--out-md")
     args = ap.parse_args()
     if args.summarize:
         return summarize(args.summarize, args.summary_layer, args.out_md)
+    if args.stream_probe:
+        return stream_probe()
     if args.gpus != 1:
         print("bench.py: this build measures one GPU only (the attention op has no cross-GPU "
               "exchange; every box here has one GPU). Run with --gpus 1.", file=sys.stderr)
@@ -351,6 +356,48 @@ def mfma_ceiling(stream, sptr, iters=6000, reps=20, warm=40):
         ms = statistics.median(a.elapsed_time(b) for a, b in evs)
         res[f"{tag}_tflops"] = round(n * 32768.0 / (ms * 1e-3) / 1e12, 1)
     return res
+
+
+def stream_probe(iters=4000, reps=5):
+    """Cycles per MFMA of the synthetic instruction streams (gptoss_attn_stream_probe), as a markdown table.  A launch
+    of the MFMA-only stream at the same occupancy gives the time of 32 matrix-pipe cycles (the pipe is busy throughout),
+    so cycles per MFMA of a mix = 32 x its time / that time; operands are zero, so the power limit plays no part."""
+    import torch
+    from oregon_gpt_oss_patching_amd import _lib
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    stream = torch.cuda.current_stream(dev)
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    sink = torch.empty(768 * cus, dtype=torch.float32, device=dev)
+
+    def timed(mix, waves):
+        def launch():
+            n = lib.gptoss_attn_stream_probe(mix, waves, iters, sink.data_ptr(), sink.numel(), stream.cuda_stream)
+            assert n > 0, n
+        for _ in range(3):
+            launch()
+        evs = []
+        for _ in range(reps):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(stream)
+            launch()
+            e1.record(stream)
+            evs.append((e0, e1))
+        torch.cuda.synchronize()
+        return statistics.median(a.elapsed_time(b) for a, b in evs)
+
+    names = ["MFMAs only", "forward, every MFMA followed by its share of the softmax", "forward, the order a compiler gives a tile",
+             "dQ, uniform", "dQ, the compiler's order", "dK/dV, uniform"]
+    base = {w: timed(0, w) / w for w in (1, 2, 3)}      # ms per wavefront's worth of MFMAs on a saturated pipe
+    print("| instruction mix | 1 wavefront per SIMD | 2 | 3 |")
+    print("|---|---|---|---|")
+    for mix, name in enumerate(names):
+        cells = []
+        for w in (1, 2, 3):
+            ms = timed(mix, w) / w
+            cyc = 32.0 * ms / base[w] if mix else 32.0 * (ms * w) / (base[1] * w)
+            cells.append(f"{cyc:.1f} cycles per MFMA ({100.0 * 32.0 / cyc:.0f} % of the matrix pipe)")
+        print(f"| {name} | " + " | ".join(cells) + " |")
 
 
 def config5():

@@ -240,6 +240,20 @@ int64_t gptoss_attn_mfma_rate_probe(const void *operands, size_t operand_bytes, 
                                     void *stream);
 
 /*
+ * Second measurement aid, likewise without counterpart in the reference and outside the attention path: runs a
+ * synthetic instruction stream with the instruction mix of one of the attention kernels (operands in registers,
+ * all zero, so the part's power limit plays no part), one workgroup per compute unit with `waves_per_simd`
+ * (1 to 3) wavefronts per SIMD, `iters` passes of 48 MFMAs per wavefront.  `mix`: 0 = MFMAs only, 1 = the forward's
+ * mix with every MFMA followed by its share of the vector work, 2 = the forward's work in the order a compiler
+ * gives a tile (MFMAs in clumps, the softmax between them), 3 / 4 = the same two for the dQ kernel, 5 = the
+ * dK/dV kernel's mix, uniform.  A benchmark times the launches against mix 0 to learn how many matrix-pipe cycles
+ * per MFMA such a kernel needs at best on this part.  `sink`: one float per thread (at least 256 * waves_per_simd *
+ * compute units).  Returns the number of MFMA instructions the launch executes, or a negative value as for
+ * gptoss_attn_mfma_rate_probe.
+ */
+int64_t gptoss_attn_stream_probe(int mix, int waves_per_simd, int iters, float *sink, size_t sink_floats, void *stream);
+
+/*
  * Host-only argument check used by every entry point; `need_bwd` != 0 also
  * requires the backward tensors.  Callable without a GPU.
  */

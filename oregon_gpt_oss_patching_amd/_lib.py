@@ -29,6 +29,7 @@ EXPORTS = (
     "gptoss_attn_bwd_static",
     "gptoss_attn_static_scratch_bytes",
     "gptoss_attn_mfma_rate_probe",
+    "gptoss_attn_stream_probe",
 )
 
 
@@ -95,6 +96,9 @@ def load() -> ctypes.CDLL:
         lib.gptoss_attn_mfma_rate_probe.restype = ctypes.c_int64
         lib.gptoss_attn_mfma_rate_probe.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p,
                                                     ctypes.c_size_t, ctypes.c_void_p]
+        lib.gptoss_attn_stream_probe.restype = ctypes.c_int64
+        lib.gptoss_attn_stream_probe.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_size_t,
+                                                 ctypes.c_void_p]
         for name in ("gptoss_attn_fwd", "gptoss_attn_bwd_preprocess", "gptoss_attn_bwd_dkdv",
                      "gptoss_attn_bwd_dq", "gptoss_attn_bwd", "gptoss_attn_bwd_static"):
             fn = getattr(lib, name)

@@ -254,6 +254,19 @@ int64_t q_outer_grid(const KArgs &a, int hpb, int qb) {
     return (int64_t)a.G * n_hc * a.B * ((a.Sq + bm - 1) / bm);
 }
 
+// one launch of a synthetic instruction stream (mfma_rate.h): one workgroup per compute unit
+template <int MIX>
+int64_t launch_stream_probe(int waves_per_simd, int iters, float *sink, hipStream_t st) {
+    const void *fn = reinterpret_cast<const void *>(stream_probe_kernel<MIX>);
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kStreamProbeLdsBytes);
+    if (e != hipSuccess) return -static_cast<int64_t>(e) - 1000;
+    const int blocks = compute_units();
+    void *args[] = {&sink, &iters};
+    e = hipLaunchKernel(fn, dim3((unsigned)blocks), dim3(256u * waves_per_simd), args, kStreamProbeLdsBytes, st);
+    if (e != hipSuccess) return -static_cast<int64_t>(e) - 1000;
+    return (int64_t)blocks * 4 * waves_per_simd * iters * kStreamProbeMfmas;     // MFMA instructions the launch executes
+}
+
 }  // namespace
 
 extern "C" {
@@ -485,6 +498,20 @@ int64_t gptoss_attn_mfma_rate_probe(const void *operands, size_t operand_bytes, 
                                          static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return -static_cast<int64_t>(e) - 1000;
     return blocks * 4 * (int64_t)iters * kMfmaRatePerIter;      // MFMA instructions the launch executes
+}
+
+int64_t gptoss_attn_stream_probe(int mix, int waves_per_simd, int iters, float *sink, size_t sink_floats, void *stream) {
+    if (!sink || iters <= 0 || mix < 0 || mix >= kStreamMixes || waves_per_simd < 1 || waves_per_simd > 3) return GPTOSS_ATTN_ERR_SHAPE;
+    if ((size_t)compute_units() * 256 * waves_per_simd > sink_floats) return GPTOSS_ATTN_ERR_SHAPE;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (mix) {
+        case kStreamMfmaOnly: return launch_stream_probe<kStreamMfmaOnly>(waves_per_simd, iters, sink, st);
+        case kStreamFwdUniform: return launch_stream_probe<kStreamFwdUniform>(waves_per_simd, iters, sink, st);
+        case kStreamFwdClumped: return launch_stream_probe<kStreamFwdClumped>(waves_per_simd, iters, sink, st);
+        case kStreamDqUniform: return launch_stream_probe<kStreamDqUniform>(waves_per_simd, iters, sink, st);
+        case kStreamDqClumped: return launch_stream_probe<kStreamDqClumped>(waves_per_simd, iters, sink, st);
+        default: return launch_stream_probe<kStreamDkdvUniform>(waves_per_simd, iters, sink, st);
+    }
 }
 
 }  // extern "C"

@@ -241,3 +241,15 @@ def test_mfma_rate_probe_refuses_bad_arguments_on_the_host():
     assert lib.gptoss_attn_mfma_rate_probe(ctypes.c_void_p(256), 8, 10, ctypes.c_void_p(256), 1 << 30, None) < 0     # under 16 bytes
     assert lib.gptoss_attn_mfma_rate_probe(ctypes.c_void_p(264), 1024, 10, ctypes.c_void_p(256), 1 << 30, None) < 0  # misaligned
     assert lib.gptoss_attn_mfma_rate_probe(ctypes.c_void_p(256), 1024, 0, ctypes.c_void_p(256), 1 << 30, None) < 0   # no passes
+
+
+def test_stream_probe_refuses_bad_arguments_on_the_host():
+    """The second measurement aid checks its arguments before it touches the device."""
+    lib = _lib.load()
+    ok_sink, many = ctypes.c_void_p(256), 1 << 30
+    assert lib.gptoss_attn_stream_probe(0, 2, 10, None, many, None) < 0            # no sink
+    assert lib.gptoss_attn_stream_probe(6, 2, 10, ok_sink, many, None) < 0         # no such mix
+    assert lib.gptoss_attn_stream_probe(-1, 2, 10, ok_sink, many, None) < 0
+    assert lib.gptoss_attn_stream_probe(0, 0, 10, ok_sink, many, None) < 0         # wavefronts per SIMD: 1 to 3
+    assert lib.gptoss_attn_stream_probe(0, 4, 10, ok_sink, many, None) < 0
+    assert lib.gptoss_attn_stream_probe(0, 2, 0, ok_sink, many, None) < 0          # no passes

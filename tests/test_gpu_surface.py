@@ -369,3 +369,24 @@ def test_mfma_rate_probe_runs_and_counts_its_mfmas():
     assert n == 2 * cus * 4 * 50 * 16
     assert bool(torch.isfinite(sink).all())
     assert lib.gptoss_attn_mfma_rate_probe(ops.data_ptr(), ops.numel() * 2, 50, sink.data_ptr(), 100, None) < 0   # sink too small
+
+
+def test_stream_probe_runs_every_mix_and_counts_its_mfmas():
+    """Every synthetic instruction stream launches at 1, 2 and 3 wavefronts per SIMD, returns the number of MFMAs it
+    executes (48 per pass and wavefront, one workgroup per compute unit) and leaves the same finite number in every
+    thread's sink slot (its operands are zero: 0 for the MFMA-only stream, a count of exp2(0) terms for the others);
+    a sink that is too small is refused."""
+    from oregon_gpt_oss_patching_amd import _lib
+    lib = _lib.load()
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    sink = torch.full((768 * cus,), float("nan"), dtype=torch.float32, device=DEV)
+    for mix in range(6):
+        for waves in (1, 2, 3):
+            sink.fill_(float("nan"))
+            n = lib.gptoss_attn_stream_probe(mix, waves, 7, sink.data_ptr(), sink.numel(), torch.cuda.current_stream().cuda_stream)
+            torch.cuda.synchronize()
+            assert n == cus * 4 * waves * 7 * 48, (mix, waves, n)
+            got = sink[:256 * waves * cus]
+            assert torch.isfinite(got).all() and (got == got[0]).all() and (mix != 0 or got[0] == 0), (mix, waves, got[0].item())
+            assert torch.isnan(sink[256 * waves * cus:]).all()           # nothing written past the launch's own threads
+    assert lib.gptoss_attn_stream_probe(0, 3, 7, sink.data_ptr(), 100, None) < 0
