@@ -14,6 +14,7 @@
 #include "attn_f32.h"
 #include "attn_fwd.h"
 #include "attn_fwd_pipe.h"
+#include "attn_fwd_window.h"
 #include "mfma_rate.h"
 
 using namespace gptoss;
@@ -141,6 +142,19 @@ bool fwd_pipe_route(const gptoss_attn_params *p) {
            !p->q_offset_dev && p->Sq == p->Skv && p->Sq % kTile == 0 && (p->H / p->G) % 4 == 0;
 }
 
+// The one-pass forward of sliding-window layers (attn_fwd_window.h): a window of 32, 64, 96 or 128 keys on plain
+// self-attention rows (no offset, no packed rows; right-padded batch rows are fine) whose padded length is a
+// multiple of 32, all four wavefronts of a workgroup with a head of their own.
+bool fwd_window_route(const gptoss_attn_params *p) {
+    const int w = effective_window(p);
+    // lane offsets are 32-bit: up to 160 rows of K / V, 32 of Q and O; the grid's y and z dimensions end at 65535
+    const int64_t row_limit = (int64_t)1 << 22;
+    if (p->k_stride.s >= row_limit || p->v_stride.s >= row_limit || p->q_stride.s >= row_limit || p->o_stride.s >= row_limit) return false;
+    if ((int64_t)(p->H / p->G / 4) * p->B > 65535 || p->Sq / 32 > 65535) return false;
+    return p->dtype == GPTOSS_ATTN_BF16 && w >= 32 && w <= 128 && w % 32 == 0 && !p->doc_start &&
+           p->q_offset == 0 && !p->q_offset_dev && p->Sq == p->Skv && p->Sq % 32 == 0 && (p->H / p->G) % 4 == 0;
+}
+
 // workgroups of four independent wavefronts for the float32 kernels
 int64_t f32_grid(int64_t waves) { return (waves + 3) / 4; }
 
@@ -153,6 +167,15 @@ int launch(Kernel kernel, int64_t workgroups, int threads, hipStream_t st, const
     void *args[] = {const_cast<KArgs *>(&a)};
     const hipError_t e = hipLaunchKernel(reinterpret_cast<const void *>(kernel), dim3((unsigned)workgroups), dim3((unsigned)threads),
                                          args, dynamic_lds, st);
+    return e == hipSuccess ? GPTOSS_ATTN_OK : static_cast<int>(e);
+}
+
+// The same for a three-dimensional grid of 256-thread workgroups (the caller has checked the y and z limits).
+template <typename Kernel>
+int launch3(Kernel kernel, dim3 grid, hipStream_t st, const KArgs &a) {
+    if (grid.x == 0 || grid.y == 0 || grid.z == 0 || grid.y > 65535 || grid.z > 65535) return GPTOSS_ATTN_ERR_SHAPE;
+    void *args[] = {const_cast<KArgs *>(&a)};
+    const hipError_t e = hipLaunchKernel(reinterpret_cast<const void *>(kernel), grid, dim3(256), args, 0, st);
     return e == hipSuccess ? GPTOSS_ATTN_OK : static_cast<int>(e);
 }
 
@@ -351,6 +374,15 @@ int gptoss_attn_fwd(const gptoss_attn_params *p, void *stream) {
         return launch(attn_f32_fwd_kernel, f32_grid((int64_t)a.B * a.H * ((a.Sq + 31) / 32)), 256, st, a);
     const int hpb = hpb_for(a.r), qb = query_blocks_for(a.window);
     const int64_t grid = q_outer_grid(a, hpb, qb);
+    if (fwd_window_route(p)) {
+        const dim3 wgrid((unsigned)a.G, (unsigned)((a.r / 4) * a.B), (unsigned)(a.Sq / 32));
+        switch (a.window / 32) {
+            case 1: return launch3(attn_fwd_window_kernel<1>, wgrid, st, a);
+            case 2: return launch3(attn_fwd_window_kernel<2>, wgrid, st, a);
+            case 3: return launch3(attn_fwd_window_kernel<3>, wgrid, st, a);
+            default: return launch3(attn_fwd_window_kernel<4>, wgrid, st, a);
+        }
+    }
     if (fwd_pipe_route(p)) return a.seqlens ? launch(attn_fwd_pipe_kernel<true>, grid, 256, st, a) : launch(attn_fwd_pipe_kernel<false>, grid, 256, st, a);
 #define GPTOSS_LAUNCH_FWD(HPB, QB) launch(attn_fwd_kernel<HPB, QB>, grid, 256, st, a)
     if (qb == 2) return hpb == 4 ? GPTOSS_LAUNCH_FWD(4, 2) : hpb == 2 ? GPTOSS_LAUNCH_FWD(2, 2) : GPTOSS_LAUNCH_FWD(1, 2);

@@ -381,3 +381,67 @@ def test_pipelined_forward_right_padded_rows(A, b, h, g, s, lens):
         assert (o[i, n:] == 0).all()
         assert torch.equal(lse[i, :, n:], lse_ref[i, :, n:])                         # the sink logit (through log2 and back)
         assert (lse[i, :, n:] - sinks.float().view(h, 1)).abs().max().item() <= 1e-6 if n < s else True
+
+
+@pytest.mark.parametrize("b,h,g,s,w", [
+    (1, 8, 2, 64, 32),          # two query blocks: the first is all "edge" (its window would start before key 0)
+    (1, 8, 2, 160, 128),        # one block beyond the edge blocks
+    (2, 16, 4, 192, 64),
+    (3, 32, 8, 1024, 96),
+    (2, 8, 1, 96, 64),          # a single KV head
+    (1, 64, 8, 4096, 128),      # config 2's sliding-window layer
+])
+def test_one_pass_window_forward_vs_the_general_forward_kernel(A, b, h, g, s, w):
+    """Sliding-window layers with a window of 32 / 64 / 96 / 128 keys take attn_fwd_window_kernel (all of a query block's
+    logits in registers, the row maximum known before the first exponential, first and last key block merged); the
+    same problem with a doc_start array that says "one document per row" takes attn_fwd_kernel (online softmax).  The
+    weights are rounded to bf16 relative to different references (the final maximum here, the running one there), so O
+    agrees to about two bf16 roundings and lse to a few units of its last fp32 place; against the eager oracle the two
+    are equally good.  Every run gives the same bits."""
+    print(f"case B={b} H={h} G={g} S={s} W={w}", flush=True)
+    q, k, v, sinks, _ = (t.to(DEV) for t in E.make_inputs(2300 + s + w, b, h, g, s, 64, torch.bfloat16))
+    one_document = torch.zeros(b, s, dtype=torch.int32, device=DEV)
+    o_ref, lse_ref = A.attention_forward(q, k, v, sinks, SCALE, w, doc_start=one_document)
+    o, lse = A.attention_forward(q, k, v, sinks, SCALE, w)
+    torch.cuda.synchronize()
+    assert torch.isfinite(o.float()).all() and torch.isfinite(lse).all()
+    assert (lse - lse_ref).abs().max().item() <= 1e-5
+    err = (o.float() - o_ref.float()).abs()
+    assert (err <= 2.0 ** -6 * o_ref.float().abs() + 2.0 ** -9).all(), err.max().item()
+    if s <= 1024:
+        qc, kc, vc, sc = q.float().cpu(), k.float().cpu(), v.float().cpu(), sinks.float().cpu()
+        want = E.eager_attention(qc, kc, vc, sc, SCALE, w)
+        want_lse = E.logsumexp_rows(qc, kc, sc, SCALE, w)
+        e_new, e_gen = (o.float().cpu() - want).abs(), (o_ref.float().cpu() - want).abs()
+        assert e_new.max().item() <= 1.05 * e_gen.max().item() + 1e-6
+        assert e_new.pow(2).mean().sqrt().item() <= 1.05 * e_gen.pow(2).mean().sqrt().item()
+        assert (lse.cpu() - want_lse).abs().max().item() <= 2e-5
+    for rep in range(3):
+        o2, lse2 = A.attention_forward(q, k, v, sinks, SCALE, w)
+        torch.cuda.synchronize()
+        assert torch.equal(o, o2) and torch.equal(lse, lse2), rep
+
+
+@pytest.mark.parametrize("b,h,g,s,w,lens", [
+    (5, 16, 4, 1088, 128, [1088, 1, 577, 1024, 64]),   # a whole row, one token, an end inside a block, on a block boundary, inside the edge blocks
+    (3, 32, 8, 256, 64, [65, 192, 0]),                 # a row with nothing in it
+])
+def test_one_pass_window_forward_right_padded_rows(A, b, h, g, s, w, lens):
+    """Right-padded batch rows through attn_fwd_window_kernel: the query block that holds a row's end gives its rows
+    of padding weights of zero, blocks past the end only write their result.  Against the general kernel: rows that
+    exist agree as in the unpadded case, rows that do not are exactly O = 0 with the same lse bits (the sink logit)."""
+    print(f"case B={b} H={h} G={g} S={s} W={w} lens={lens}", flush=True)
+    q, k, v, sinks, _ = (t.to(DEV) for t in E.make_inputs(2500 + s, b, h, g, s, 64, torch.bfloat16))
+    one_document = torch.zeros(b, s, dtype=torch.int32, device=DEV)
+    o_ref, lse_ref = A.attention_forward(q, k, v, sinks, SCALE, w, 0, lens, doc_start=one_document)
+    o, lse = A.attention_forward(q, k, v, sinks, SCALE, w, 0, lens)
+    torch.cuda.synchronize()
+    assert torch.isfinite(o.float()).all() and torch.isfinite(lse).all()
+    assert (lse - lse_ref).abs().max().item() <= 1e-5
+    err = (o.float() - o_ref.float()).abs()
+    assert (err <= 2.0 ** -6 * o_ref.float().abs() + 2.0 ** -9).all(), err.max().item()
+    for i, n in enumerate(lens):
+        assert (o[i, n:] == 0).all()
+        assert torch.equal(lse[i, :, n:], lse_ref[i, :, n:])
+        if n < s:
+            assert (lse[i, :, n:] - sinks.float().view(h, 1)).abs().max().item() <= 1e-6
