@@ -117,7 +117,8 @@ __global__ __launch_bounds__(256, 3) void attn_fwd_window_kernel(const KArgs a) 
     const TileLaneOffsets lo = make_tile_offsets(lane);
     const int x = l32 - 4 * half;                  // register i of a block holds key rc(i) + 4 half: "key <= row" is rc(i) <= x
 
-    __syncthreads();                               // K and V have landed (the compiler waits for the copies in front of a barrier)
+    wait_vmcnt<0>();                               // this wavefront's copies of K and V (and its Q rows) have landed ...
+    __syncthreads();                               // ... and everybody else's
 
     // S^T = K Q^T for all NH blocks: lane = query row l32, register i of block h = key 32 h + rc(i) + 4 half
     f32x16 s[NH];

@@ -54,3 +54,12 @@ def test_three_wavefronts_per_simd_and_no_scratch(assembly):
 def test_maxima_are_compiler_made(assembly):
     assert "v_max3_f32" in assembly
     assert "#APP" not in assembly          # no inline assembly in this kernel
+
+
+def test_copies_are_waited_for_in_front_of_the_first_barrier(assembly):
+    for kernel in assembly.split(".end_amdhsa_kernel")[:4]:
+        lines = [x.strip() for x in kernel.split("\n")]
+        first_barrier = next(i for i, x in enumerate(lines) if x.startswith("s_barrier"))
+        last_copy = max(i for i, x in enumerate(lines) if x.startswith("global_load_lds_dwordx4"))
+        assert last_copy < first_barrier
+        assert any(re.match(r"s_waitcnt vmcnt\(0\)", x) for x in lines[last_copy:first_barrier])
