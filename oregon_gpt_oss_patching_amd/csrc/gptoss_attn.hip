@@ -375,7 +375,11 @@ int gptoss_attn_fwd(const gptoss_attn_params *p, void *stream) {
     const int hpb = hpb_for(a.r), qb = query_blocks_for(a.window);
     const int64_t grid = q_outer_grid(a, hpb, qb);
     if (fwd_window_route(p)) {
-        const dim3 wgrid((unsigned)a.G, (unsigned)((a.r / 4) * a.B), (unsigned)(a.Sq / 32));
+        // two 32-row query blocks per workgroup (K / V rows staged once for both) where that still leaves every compute
+        // unit several rounds of workgroups, else one
+        const int64_t pairs = (int64_t)a.G * (a.r / 4) * a.B * ((a.Sq + 63) / 64);
+        const bool by_pairs = a.Sq > 32 && pairs >= 8 * (int64_t)compute_units();
+        const dim3 wgrid((unsigned)a.G, (unsigned)((a.r / 4) * a.B), (unsigned)(by_pairs ? (a.Sq + 63) / 64 : a.Sq / 32));
         switch (a.window / 32) {
             case 1: return launch3(attn_fwd_window_kernel<1>, wgrid, st, a);
             case 2: return launch3(attn_fwd_window_kernel<2>, wgrid, st, a);

@@ -445,3 +445,33 @@ def test_one_pass_window_forward_right_padded_rows(A, b, h, g, s, w, lens):
         assert torch.equal(lse[i, :, n:], lse_ref[i, :, n:])
         if n < s:
             assert (lse[i, :, n:] - sinks.float().view(h, 1)).abs().max().item() <= 1e-6
+
+
+@pytest.mark.parametrize("b,h,g,s,w,lens", [
+    (4, 64, 8, 2048, 128, None),                       # 2048 pairs of query blocks
+    (4, 64, 8, 2080, 128, None),                       # an odd number of query blocks: the last workgroup of a row has one
+    (4, 64, 8, 2048, 64, [2048, 33, 1000, 1984]),      # ends in a pair's second block, in its first, on a pair boundary
+    (8, 32, 8, 4096, 96, None),
+])
+def test_one_pass_window_forward_two_query_blocks_per_workgroup(A, b, h, g, s, w, lens):
+    """Problems with enough work for several rounds of workgroups per compute unit are launched with two 32-row query
+    blocks per workgroup of attn_fwd_window_kernel: the staged K / V rows serve both, the first block's results leave
+    through the 32 staged rows that the second block does not need.  Compared with the general kernel as in the
+    one-block case (which the smaller shapes of the tests above take)."""
+    print(f"case B={b} H={h} G={g} S={s} W={w} lens={lens}", flush=True)
+    q, k, v, sinks, _ = (t.to(DEV) for t in E.make_inputs(2700 + s + w, b, h, g, s, 64, torch.bfloat16))
+    one_document = torch.zeros(b, s, dtype=torch.int32, device=DEV)
+    o_ref, lse_ref = A.attention_forward(q, k, v, sinks, SCALE, w, 0, lens, doc_start=one_document)
+    o, lse = A.attention_forward(q, k, v, sinks, SCALE, w, 0, lens)
+    torch.cuda.synchronize()
+    assert torch.isfinite(o.float()).all() and torch.isfinite(lse).all()
+    assert (lse - lse_ref).abs().max().item() <= 1e-5
+    err = (o.float() - o_ref.float()).abs()
+    assert (err <= 2.0 ** -6 * o_ref.float().abs() + 2.0 ** -9).all(), err.max().item()
+    if lens is not None:
+        for i, n in enumerate(lens):
+            assert (o[i, n:] == 0).all()
+            assert torch.equal(lse[i, :, n:], lse_ref[i, :, n:])
+    o2, lse2 = A.attention_forward(q, k, v, sinks, SCALE, w, 0, lens)
+    torch.cuda.synchronize()
+    assert torch.equal(o, o2) and torch.equal(lse, lse2)
