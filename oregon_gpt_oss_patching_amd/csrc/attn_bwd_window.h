@@ -145,7 +145,7 @@ __global__ __launch_bounds__(WinCfg::NWAVES * 64, 1) void attn_bwd_window_kernel
         const bf16 *orow = a.o + (int64_t)b * a.os.b + (int64_t)(g * a.r) * a.os.h + stat_row0 * a.os.s + 32 * hr;
         const bf16 *grow = a.d_o + (int64_t)b * a.dos.b + (int64_t)(g * a.r) * a.dos.h + stat_row0 * a.dos.s + 32 * hr;
         const float *lrow = a.lse + ((int64_t)b * a.H + (int64_t)g * a.r) * a.Sq + stat_row0;
-        auto prefetch = [&](WinPos &pos) {
+        auto prefetch = [&](WinPos &pos) __attribute__((always_inline)) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 pre_o[j] = *reinterpret_cast<const u32x4 *>(orow + 8 * j);
@@ -166,7 +166,7 @@ __global__ __launch_bounds__(WinCfg::NWAVES * 64, 1) void attn_bwd_window_kernel
             }
         };
         // row statistics of the prefetched rows into stage `stage`; dSinks terms of own rows
-        auto statistics = [&](const WinPos &pos, int stage) {
+        auto statistics = [&](const WinPos &pos, int stage) __attribute__((always_inline)) {
             typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
             float acc = 0.0f;
 #pragma unroll
@@ -207,18 +207,24 @@ __global__ __launch_bounds__(WinCfg::NWAVES * 64, 1) void attn_bwd_window_kernel
         p_stat.step(a.r);
         if (n_it > 1) prefetch(p_pre);
 
+        // the fragment offsets with the address of the dS buffer at hand folded in (they are the only copy of the lane
+        // offsets this wavefront keeps: its other reads go relative to the same address)
+        TileLaneOffsets lo_ds = tile_offsets_at(lo, ds_base);
+        uint32_t lo_ds_at = ds_base;
         // dQ rows 32*hh.. of the tile at `pos` from the dS tile at LDS address ds_tile
-        auto helper_dq = [&](uint32_t ds_tile, const WinPos &pos) {
+        auto helper_dq = [&](uint32_t ds_tile, const WinPos &pos) __attribute__((always_inline)) {
             f32x16 acc[2];
 #pragma unroll
             for (int db = 0; db < 2; ++db)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) acc[db][i] = 0.0f;
+            tile_offsets_move(lo_ds, ds_tile - lo_ds_at);      // the lane offsets follow the dS buffer (one add each, immediates from there)
+            lo_ds_at = ds_tile;
 #pragma unroll
             for (int p = 0; p < 3; ++p)
 #pragma unroll
                 for (int kk = 0; kk < 4; ++kk) {
-                    const bf16x8 ads = ofrag_tr(ds_tile + p * kStageTileBytes, lo, kk >> 1, kk & 1, hh);
+                    const bf16x8 ads = ofrag_tr(p * kStageTileBytes, lo_ds, kk >> 1, kk & 1, hh);
 #pragma unroll
                     for (int db = 0; db < 2; ++db) acc[db] = mfma_bf16(kfr[p][kk][db], ads, acc[db]);
                 }
@@ -228,12 +234,12 @@ __global__ __launch_bounds__(WinCfg::NWAVES * 64, 1) void attn_bwd_window_kernel
             store_rows32(out_stage, acc, a.scale, row0, a.dqs.s, a.Sq - r0, lane);
             __builtin_amdgcn_wave_barrier();
         };
-        auto reload = [&](auto slot_tag) {
+        auto reload = [&](auto slot_tag) __attribute__((always_inline)) {
             constexpr int P = decltype(slot_tag)::value;
 #pragma unroll
             for (int kk = 0; kk < 4; ++kk)
 #pragma unroll
-                for (int db = 0; db < 2; ++db) kfr[P][kk][db] = ofrag_tr(transit_base, lo, kk >> 1, kk & 1, db);
+                for (int db = 0; db < 2; ++db) kfr[P][kk][db] = ofrag_tr(transit_base - lo_ds_at, lo_ds, kk >> 1, kk & 1, db);
         };
 
         WinPos cur{t0, 0};
@@ -273,7 +279,7 @@ __global__ __launch_bounds__(WinCfg::NWAVES * 64, 1) void attn_bwd_window_kernel
     int my_kt = tile_of_slot(pair, t0);                        // key tile held (negative: none yet)
     bf16x8 kf[1][4], vf[1][4];
     f32x16 dk[1][2], dv[1][2];
-    auto clear_acc = [&]() {
+    auto clear_acc = [&]() __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) { dk[0][0][i] = dk[0][1][i] = 0.0f; dv[0][0][i] = dv[0][1][i] = 0.0f; }
     };
@@ -299,7 +305,7 @@ __global__ __launch_bounds__(WinCfg::NWAVES * 64, 1) void attn_bwd_window_kernel
     auto seam_slot = [&](int seam, int tile, int side) {
         return a.boundary_partial + (((((int64_t)b * a.G + g) * (n_chunks - 1) + seam) * 2 + tile) * 2 + side) * (2 * kTile * kD);
     };
-    auto store_share = [&](float *dst) {
+    auto store_share = [&](float *dst) __attribute__((always_inline)) {
         // unscaled fp32 sums; lane = key row, register i of block dblk = column 32*dblk + crow(i, half),
         // four consecutive columns per 16-byte store
         float *pk = dst + (32 * sub + l32) * kD, *pv = pk + kTile * kD;
@@ -317,7 +323,7 @@ __global__ __launch_bounds__(WinCfg::NWAVES * 64, 1) void attn_bwd_window_kernel
     };
     // dK / dV of the key tile held: written out if it is complete, left as this workgroup's share if
     // it sits on a seam, dropped if it belongs to the neighbour (recomputation mode)
-    auto flush = [&]() {
+    auto flush = [&]() __attribute__((always_inline)) {
         if (my_kt < 0) return;
         if (seam_sums) {
             if (my_kt < t0) { store_share(seam_slot(chunk - 1, my_kt - (t0 - 2), 1)); return; }
@@ -354,7 +360,7 @@ __global__ __launch_bounds__(WinCfg::NWAVES * 64, 1) void attn_bwd_window_kernel
     const bf16 *ld_tile = (w == kWaveQ)
         ? a.q + (int64_t)b * a.qs.b + (int64_t)(g * a.r) * a.qs.h + (int64_t)iss_i0 * a.qs.s
         : a.d_o + (int64_t)b * a.dos.b + (int64_t)(g * a.r) * a.dos.h + (int64_t)iss_i0 * a.dos.s;
-    auto issue = [&](int it) {
+    auto issue = [&](int it) __attribute__((always_inline)) {
         const int stage = it % NS;
         if (w == kWaveQ || w == kWaveDO) {
             char *dst = smem + (stage * 2 + (w - kWaveQ)) * kStageTileBytes;
@@ -384,7 +390,7 @@ __global__ __launch_bounds__(WinCfg::NWAVES * 64, 1) void attn_bwd_window_kernel
             ld_tile += (int64_t)kTile * lstride - (int64_t)a.r * ld_hstride;
         }
     };
-    auto issue_transit = [&](int kt) {
+    auto issue_transit = [&](int kt) __attribute__((always_inline)) {
 #pragma unroll 1
         for (int k = 0; k < 8; ++k) {
             const int rr = 8 * k + (lane >> 3);
@@ -406,9 +412,18 @@ __global__ __launch_bounds__(WinCfg::NWAVES * 64, 1) void attn_bwd_window_kernel
     // One copy of the loop body with the LDS stage as a run-time value: a body per stage (stage
     // offsets as instruction immediates) makes this kernel larger than the instruction cache.
     int stage = 0;
-    auto iterate = [&](int it) {
+    // the fragment offsets with the address of the stage at hand folded in: one add each per walk position, and every
+    // read of the position's Q and dO tiles is (register) + (immediate)
+    TileLaneOffsets lo_st = tile_offsets_at(lo, smem_base);
+    uint32_t lo_st_at = smem_base;
+    auto iterate = [&](int it) __attribute__((always_inline)) {
         const int STAGE = stage;
         stage = stage == NS - 1 ? 0 : stage + 1;
+        {
+            const uint32_t at = smem_base + STAGE * (2 * kStageTileBytes);
+            tile_offsets_move(lo_st, at - lo_st_at);
+            lo_st_at = at;
+        }
         if (w == kWaveQ || w == kWaveDO) { if (it + 1 >= n_it) wait_vmcnt<0>(); else wait_vmcnt<8>(); }
         else if (w == kWaveTransit && cur.h == 0) wait_vmcnt<0>();        // the transit copy of the key tile that starts now
         __syncthreads();
@@ -422,8 +437,8 @@ __global__ __launch_bounds__(WinCfg::NWAVES * 64, 1) void attn_bwd_window_kernel
             if (my_kt >= 0) {
 #pragma unroll
                 for (int ks = 0; ks < 4; ++ks) {
-                    kf[0][ks] = ofrag_nat(transit_base, lo, sub, ks);
-                    vf[0][ks] = ofrag_nat(transit_base + kStageTileBytes, lo, sub, ks);
+                    kf[0][ks] = ofrag_nat(transit_base - lo_st_at, lo_st, sub, ks);
+                    vf[0][ks] = ofrag_nat(transit_base + kStageTileBytes - lo_st_at, lo_st, sub, ks);
                 }
             }
             clear_acc();
@@ -440,17 +455,18 @@ __global__ __launch_bounds__(WinCfg::NWAVES * 64, 1) void attn_bwd_window_kernel
             ds_store_zero(ds_out, 0);
             ds_store_zero(ds_out, 1);
         } else {
-            const uint32_t qsm = smem_base + STAGE * (2 * kStageTileBytes), gsm = qsm + kStageTileBytes;
+            // (fragment addresses: the stage's address is in the lane offsets, the dO tile is 8 KB behind Q's)
+            const uint32_t qsm = 0u, gsm = kStageTileBytes;
             const uint32_t stat_lane = stat_base + STAGE * (2 * kTile * 4) + half * 16;
             const bool interior = (wj0 + 31 <= pos0) && (wj0 > pos1 - weff) && (wj0 + 32 <= kv_len) && (i0 + kTile - 1 <= pos1);
             int jkey[1] = {wj0 + l32};
             if (interior) {
-                dkdv_tile<false, false, 1, true>(qsm, gsm, stat_lane, lo, kf, vf, dk, dv, c, half, dead, 0u, 0, 0, 0u, jkey, ds_out);
+                dkdv_tile<false, false, 1, true>(qsm, gsm, stat_lane, lo_st, kf, vf, dk, dv, c, half, dead, 0u, 0, 0, 0u, jkey, ds_out);
             } else {
                 int dbase[1];
                 dbase[0] = (wj0 + l32 < kv_len) ? pos0 - (wj0 + l32) : -0x40000000;
                 const int row_lim = min(kTile, min(a.Sq, q_len) - i0);
-                dkdv_tile<true, false, 1, true>(qsm, gsm, stat_lane, lo, kf, vf, dk, dv, c, half, dbase, (unsigned)weff, row_lim,
+                dkdv_tile<true, false, 1, true>(qsm, gsm, stat_lane, lo_st, kf, vf, dk, dv, c, half, dbase, (unsigned)weff, row_lim,
                                                 wj0 - pos0, 0u, jkey, ds_out);
             }
         }

@@ -311,6 +311,30 @@ __device__ __forceinline__ TileLaneOffsets make_tile_offsets(int lane) {
     return o;
 }
 
+// The lane offsets with a tile's (run-time) LDS address added once, for code that reads many fragments of one tile:
+// the fragment reads then take (this register) + (immediate) and tile = 0.  The sums are hidden from the compiler,
+// which otherwise folds the block / tensor constants into the scalar tile address and pays one vector add per read.
+__device__ __forceinline__ TileLaneOffsets tile_offsets_at(const TileLaneOffsets &o, uint32_t tile) {
+    TileLaneOffsets r;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) { r.nat[ks] = tile + o.nat[ks]; asm volatile("" : "+v"(r.nat[ks])); }
+#pragma unroll
+    for (int dblk = 0; dblk < 2; ++dblk)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) { r.tr[dblk][t] = tile + o.tr[dblk][t]; asm volatile("" : "+v"(r.tr[dblk][t])); }
+    return r;
+}
+
+// moves such offsets from one tile address to another (delta = new address - old address, modulo 2^32)
+__device__ __forceinline__ void tile_offsets_move(TileLaneOffsets &r, uint32_t delta) {
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) { r.nat[ks] += delta; asm volatile("" : "+v"(r.nat[ks])); }
+#pragma unroll
+    for (int dblk = 0; dblk < 2; ++dblk)
+#pragma unroll
+        for (int t = 0; t < 2; ++t) { r.tr[dblk][t] += delta; asm volatile("" : "+v"(r.tr[dblk][t])); }
+}
+
 // natural fragment of 32-row block `blk`; `tile` = LDS byte address of the tile
 __device__ __forceinline__ bf16x8 ofrag_nat(uint32_t tile, const TileLaneOffsets &o, int blk, int ks) {
     return as_bf16x8(lds_load128(tile + o.nat[ks], blk * 32 * kRowBytes));
