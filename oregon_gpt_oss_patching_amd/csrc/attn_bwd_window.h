@@ -207,10 +207,6 @@ __global__ __launch_bounds__(WinCfg::NWAVES * 64, 1) void attn_bwd_window_kernel
         p_stat.step(a.r);
         if (n_it > 1) prefetch(p_pre);
 
-        // the fragment offsets with the address of the dS buffer at hand folded in (they are the only copy of the lane
-        // offsets this wavefront keeps: its other reads go relative to the same address)
-        TileLaneOffsets lo_ds = tile_offsets_at(lo, ds_base);
-        uint32_t lo_ds_at = ds_base;
         // dQ rows 32*hh.. of the tile at `pos` from the dS tile at LDS address ds_tile
         auto helper_dq = [&](uint32_t ds_tile, const WinPos &pos) __attribute__((always_inline)) {
             f32x16 acc[2];
@@ -218,13 +214,11 @@ __global__ __launch_bounds__(WinCfg::NWAVES * 64, 1) void attn_bwd_window_kernel
             for (int db = 0; db < 2; ++db)
 #pragma unroll
                 for (int i = 0; i < 16; ++i) acc[db][i] = 0.0f;
-            tile_offsets_move(lo_ds, ds_tile - lo_ds_at);      // the lane offsets follow the dS buffer (one add each, immediates from there)
-            lo_ds_at = ds_tile;
 #pragma unroll
             for (int p = 0; p < 3; ++p)
 #pragma unroll
                 for (int kk = 0; kk < 4; ++kk) {
-                    const bf16x8 ads = ofrag_tr(p * kStageTileBytes, lo_ds, kk >> 1, kk & 1, hh);
+                    const bf16x8 ads = ofrag_tr(ds_tile + p * kStageTileBytes, lo, kk >> 1, kk & 1, hh);
 #pragma unroll
                     for (int db = 0; db < 2; ++db) acc[db] = mfma_bf16(kfr[p][kk][db], ads, acc[db]);
                 }
@@ -239,7 +233,7 @@ __global__ __launch_bounds__(WinCfg::NWAVES * 64, 1) void attn_bwd_window_kernel
 #pragma unroll
             for (int kk = 0; kk < 4; ++kk)
 #pragma unroll
-                for (int db = 0; db < 2; ++db) kfr[P][kk][db] = ofrag_tr(transit_base - lo_ds_at, lo_ds, kk >> 1, kk & 1, db);
+                for (int db = 0; db < 2; ++db) kfr[P][kk][db] = ofrag_tr(transit_base, lo, kk >> 1, kk & 1, db);
         };
 
         WinPos cur{t0, 0};
